@@ -1,0 +1,169 @@
+/*
+ * pith_hip.h — flat C ABI of libpith_hip.so: MI355X (gfx950) kernels for PithTrain's
+ * context-parallel ring-attention hot path.
+ *
+ * Conventions (all entry points):
+ *   - return 0 (PITH_OK) on success, a negative PITH_ERR_* code otherwise; the text of the
+ *     last error of the calling thread is available from pith_last_error();
+ *   - every pointer is a borrowed DEVICE pointer; the library allocates and frees nothing and
+ *     keeps no state between calls; calls only enqueue work on `stream` (a hipStream_t passed
+ *     as void*, NULL = the default stream) and never synchronise the device;
+ *   - activations are bf16 in BSHD order, x[b, s, h, d] at  b*batch_stride + (s*H + h)*D + d
+ *     (strides in ELEMENTS; the row stride H*D and head stride D are implied, which is what
+ *     the reference asserts with .is_contiguous(); the separate batch stride lets a caller
+ *     pass a slice along S without copying);
+ *   - LSE and delta are fp32 in BHS order, lse[b, h, s] at  b*bs + h*hs + s  with both
+ *     strides given so that a row sub-range of a [B,H,S] tensor can be addressed in place;
+ *   - LSE is base-2 (log2 of the softmax denominator in the scaled-score domain) unless a
+ *     `base` field says otherwise.
+ *
+ * Reference interface replaced (paths relative to the PithTrain tree):
+ *   pithtrain/operators/mla/triton.py:552-603        _mla_fwd / _mla_bwd_preprocess / _mla_bwd_dk_dv / _mla_bwd_dq
+ *   pithtrain/operators/ring_attention/standard.py:91-93,134-153   flash-attn _flash_attn_forward / _flash_attn_backward call sites
+ *   pithtrain/operators/ring_attention/mla.py:27-40  _online_softmax_combine_log2
+ *   pithtrain/operators/ring_attention/standard.py:53-66  _online_softmax_combine
+ */
+#ifndef PITH_HIP_H
+#define PITH_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* pith_stream_t; /* hipStream_t */
+
+enum {
+  PITH_OK = 0,
+  PITH_ERR_NULL_POINTER = -1, /* a required pointer argument is NULL */
+  PITH_ERR_BAD_SHAPE = -2,    /* a size is <= 0, or sizes are inconsistent with each other */
+  PITH_ERR_BAD_DTYPE = -3,    /* a dtype / base enum is out of range */
+  PITH_ERR_UNSUPPORTED = -4,  /* valid request this build has no kernel for (head dims, causal with Sq != Skv) */
+  PITH_ERR_MISALIGNED = -5,   /* a pointer or stride breaks the 16-byte vector-access requirement */
+  PITH_ERR_LAUNCH = -6        /* the HIP runtime refused the launch */
+};
+
+enum { PITH_BF16 = 0, PITH_F32 = 1 };
+enum { PITH_BASE_2 = 0, PITH_BASE_E = 1 };
+
+/* Library version: major*10000 + minor*100 + patch. */
+int pith_version(void);
+/* Text of the last error raised on the calling thread ("" if none). Never NULL. */
+const char* pith_last_error(void);
+/* Symbolic name of an error code ("PITH_OK", "PITH_ERR_BAD_SHAPE", ...). Never NULL. */
+const char* pith_error_name(int code);
+
+/* ------------------------------------------------------------------------------------------
+ * Online-softmax combine of two partial attention results.
+ * Replaces _online_softmax_combine_log2 (ring_attention/mla.py:27-40, base 2) and
+ * _online_softmax_combine (ring_attention/standard.py:53-66, base e):
+ *     M = max(l1,l2); w1 = beta^(l1-M); w2 = beta^(l2-M)
+ *     out = (w1*out1 + w2*out2)/(w1+w2);  lse = M + log_beta(w1+w2)
+ * out1/out2 may each be bf16 or fp32 (the running accumulator of the ring is fp32, a chunk
+ * result is bf16); `out` is fp32 (what the reference's type promotion yields) or bf16 (used
+ * for the last ring step, fusing the reference's final .to(q.dtype), mla.py:78).
+ * `out` may alias out1 or out2 when the dtypes match; lse_out may alias lse1 or lse2.
+ * D must be a multiple of 8; base pointers and batch strides must keep 16-byte alignment. */
+typedef struct {
+  const void* out1;
+  const float* lse1;
+  const void* out2;
+  const float* lse2;
+  void* out;
+  float* lse_out;
+  int32_t dtype1, dtype2, dtype_out; /* PITH_BF16 | PITH_F32 */
+  int32_t base;                      /* PITH_BASE_2 | PITH_BASE_E */
+  int64_t B, S, H, D;
+  int64_t out1_bs, out2_bs, out_bs;  /* batch strides of the three O tensors, elements */
+  int64_t lse1_bs, lse1_hs;          /* batch / head strides of lse1 */
+  int64_t lse2_bs, lse2_hs;
+  int64_t lse_out_bs, lse_out_hs;
+} pith_combine_args;
+
+int pith_combine(const pith_combine_args* args, pith_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * One chunk attention forward: O = softmax(scale * Q K^T [+ causal mask]) V and the base-2 LSE.
+ * Replaces _mla_fwd (mla/triton.py:552-563; kernels :32-93 causal, :274-323 non-causal) and the
+ * _flash_attn_forward call at ring_attention/standard.py:91-93 (whose LSE is natural-log:
+ * LSE_e = LSE_2 * ln 2).
+ * q [B,Sq,Hq,Dqk], k [B,Skv,Hkv,Dqk], v [B,Skv,Hkv,Dv], o [B,Sq,Hq,Dv] bf16; lse [B,Hq,Sq] fp32.
+ * Query head h reads kv head h / (Hq/Hkv). causal != 0 masks key j > query i and needs
+ * Sq == Skv. Supported (Dqk, Dv): (64,64), (128,128), (192,128). Sq and Skv are arbitrary. */
+typedef struct {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  float* lse;
+  int64_t B, Sq, Skv, Hq, Hkv, Dqk, Dv;
+  int64_t q_bs, k_bs, v_bs, o_bs; /* batch strides, elements */
+  int64_t lse_bs, lse_hs;
+  float scale;
+  int32_t causal;
+} pith_attn_fwd_args;
+
+int pith_attn_fwd(const pith_attn_fwd_args* args, pith_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * delta[b,h,s] = sum_d fp32(o[b,s,h,d]) * fp32(dout[b,s,h,d]).
+ * Replaces _mla_bwd_preprocess (mla/triton.py:566-574; kernel :101-122). */
+typedef struct {
+  const void* o;
+  const void* dout;
+  float* delta;
+  int64_t B, S, H, D;
+  int64_t o_bs, dout_bs;
+  int64_t delta_bs, delta_hs;
+} pith_attn_delta_args;
+
+int pith_attn_bwd_delta(const pith_attn_delta_args* args, pith_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * One chunk attention backward against an EXTERNAL (ring-combined) base-2 LSE and delta:
+ *     P = exp2(scale*log2(e)*S - lse);  dV = P^T dO;  dP = dO V^T;
+ *     dS = P o (dP - delta) * scale;    dK = dS^T Q;  dQ = dS K
+ * Replaces _mla_bwd_dk_dv / _mla_bwd_dq (mla/triton.py:577-603; kernels :130-197, :205-266 and
+ * the non-causal twins :331-441) and the _flash_attn_backward call at
+ * ring_attention/standard.py:134-153.
+ * Shapes as in pith_attn_fwd_args; dout [B,Sq,Hq,Dv] bf16; lse, delta [B,Hq,Sq] fp32.
+ * dq [B,Sq,Hq,Dqk], dk [B,Skv,Hkv,Dqk], dv [B,Skv,Hkv,Dv] in dq_dtype / dkv_dtype
+ * (PITH_BF16 as the reference stores them, or PITH_F32 for a ring-level accumulator).
+ * accumulate_dq != 0 adds to the existing contents of dq instead of overwriting (the ring's
+ * `dq += dq_s`, ring_attention/mla.py:116, done in the kernel epilogue); the same for
+ * accumulate_dkv. With Hq > Hkv, dk/dv of a kv head sum over its Hq/Hkv query heads.
+ * pith_attn_bwd_dkdv ignores dq; pith_attn_bwd_dq ignores dk, dv. */
+typedef struct {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* dout;
+  const float* lse;
+  const float* delta;
+  void* dq;
+  void* dk;
+  void* dv;
+  int64_t B, Sq, Skv, Hq, Hkv, Dqk, Dv;
+  int64_t q_bs, k_bs, v_bs, dout_bs;
+  int64_t dq_bs, dk_bs, dv_bs;
+  int64_t lse_bs, lse_hs;     /* strides shared by lse and delta */
+  float scale;
+  int32_t causal;
+  int32_t dq_dtype, dkv_dtype;
+  int32_t accumulate_dq, accumulate_dkv;
+} pith_attn_bwd_args;
+
+int pith_attn_bwd_dkdv(const pith_attn_bwd_args* args, pith_stream_t stream);
+int pith_attn_bwd_dq(const pith_attn_bwd_args* args, pith_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * dst[i] = bf16(src[i]) with round-to-nearest-even, i < n. Replaces the reference's
+ * `.to(q.dtype)` on an fp32 accumulator (ring_attention/mla.py:78, standard.py:104) when the
+ * last combine did not already emit bf16. n must be a multiple of 8. */
+int pith_cast_f32_bf16(const float* src, void* dst, int64_t n, pith_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PITH_HIP_H */

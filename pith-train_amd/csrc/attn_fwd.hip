@@ -1,0 +1,279 @@
+// One chunk attention forward for gfx950: O = softmax(scale * Q K^T [+causal]) V, base-2 LSE.
+// Numerics follow pithtrain/operators/mla/triton.py:32-93 (causal) and :274-323 (non-causal):
+// fp32 scores from bf16 MFMA, P = exp2(kappa*(s - m)) in fp32, row sum from the fp32 P, P rounded
+// to bf16 for P V, O = acc / l rounded to bf16, LSE2 = log2(l) + kappa*m, kappa = scale*log2(e).
+//
+// Work split: a workgroup of 4 wavefronts owns 256 consecutive query rows of one (batch, head);
+// each wavefront owns 64 of them (two 32-wide column blocks). K/V tiles of 64 keys are staged
+// through LDS (double buffered, fetched to registers one tile ahead) and shared by the 4 waves.
+// Scores are produced TRANSPOSED, S^T = K Q^T, so that a lane holds one query column: the
+// softmax row reductions are in-lane plus one exchange with the partner lane, and P^T feeds the
+// second product O^T += V^T P^T straight from registers; V^T comes from transposing LDS reads.
+#include "attn_tiles.h"
+
+namespace pith {
+namespace {
+
+constexpr int kFwdThreads = 256;
+constexpr int kFwdWaves = 4;
+constexpr int kFwdRowsPerWave = 64;
+constexpr int kFwdBlockM = kFwdWaves * kFwdRowsPerWave;
+constexpr int kFwdBlockN = 64;
+
+struct FwdParams {
+  const __bf16* q;
+  const __bf16* k;
+  const __bf16* v;
+  __bf16* o;
+  float* lse;
+  int Sq, Skv, Hq, Hkv, group;  // group = Hq / Hkv
+  int m_tiles;
+  int64_t q_bs, k_bs, v_bs, o_bs, lse_bs, lse_hs;
+  float kappa;  // scale * log2(e)
+};
+
+template <int DQK, int DV, bool CAUSAL>
+__global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_fwd_kernel(
+    FwdParams p) {
+  constexpr int KS = DQK / 16;         // contraction steps of Q K^T
+  constexpr int DVB = DV / 32;         // 32-row blocks of O^T
+  constexpr int KP = DQK * 2 + 16;     // K tile pitch: conflict-free 16-byte row reads
+  constexpr int VP = DV * 2 + 64;      // V tile pitch: conflict-free transposing reads
+  constexpr int kKTile = kFwdBlockN * KP;
+  constexpr int kVTile = kFwdBlockN * VP;
+  __shared__ __attribute__((aligned(16))) char smem[2 * (kKTile + kVTile)];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, g = lane >> 5;
+
+  // Heaviest (latest) query tiles are scheduled first under the causal mask.
+  const int m_tile = p.m_tiles - 1 - blockIdx.x;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int hk = h / p.group;
+  const int m0 = m_tile * kFwdBlockM;
+  const int q_wave0 = m0 + wave * kFwdRowsPerWave;
+
+  const int64_t q_row_stride = (int64_t)p.Hq * DQK;
+  const int64_t k_row_stride = (int64_t)p.Hkv * DQK;
+  const int64_t v_row_stride = (int64_t)p.Hkv * DV;
+  const int64_t o_row_stride = (int64_t)p.Hq * DV;
+  const __bf16* qh = p.q + b * p.q_bs + (int64_t)h * DQK;
+  const __bf16* kh = p.k + b * p.k_bs + (int64_t)hk * DQK;
+  const __bf16* vh = p.v + b * p.v_bs + (int64_t)hk * DV;
+
+  // Q^T fragments (B operand): column = query row, slots = 8 consecutive features.
+  bf16x8 qf[2][KS];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    int row = q_wave0 + qb * 32 + c;
+    row = row < p.Sq ? row : p.Sq - 1;
+    const __bf16* src = qh + row * q_row_stride + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[qb][ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
+  }
+
+  f32x16 oacc[DVB][2];
+#pragma unroll
+  for (int i = 0; i < DVB; ++i)
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) oacc[i][qb][v] = 0.f;
+  float m_run[2] = {-INFINITY, -INFINITY};
+  float l_run[2] = {0.f, 0.f};  // this lane's share of the row sum (partner lane holds the rest)
+
+  // Number of key tiles this workgroup / this wavefront has to visit.
+  const int n_tiles_all = (p.Skv + kFwdBlockN - 1) / kFwdBlockN;
+  int n_tiles_wg = n_tiles_all, n_tiles_wave = n_tiles_all;
+  if (CAUSAL) {
+    n_tiles_wg = min(n_tiles_all, (m0 + kFwdBlockM) / kFwdBlockN);
+    n_tiles_wave = min(n_tiles_all, q_wave0 / kFwdBlockN + 1);
+  }
+
+  TileCopy<kFwdBlockN, DQK, KP, kFwdThreads> kcopy;
+  TileCopy<kFwdBlockN, DV, VP, kFwdThreads> vcopy;
+  kcopy.fetch(kh, k_row_stride, 0, p.Skv, tid);
+  vcopy.fetch(vh, v_row_stride, 0, p.Skv, tid);
+  kcopy.commit(smem, tid);
+  vcopy.commit(smem + kKTile, tid);
+  __syncthreads();
+
+  for (int t = 0; t < n_tiles_wg; ++t) {
+    const char* ktile = smem + (t & 1) * (kKTile + kVTile);
+    const char* vtile = ktile + kKTile;
+    const bool have_next = t + 1 < n_tiles_wg;
+    if (have_next) {
+      kcopy.fetch(kh, k_row_stride, (t + 1) * kFwdBlockN, p.Skv, tid);
+      vcopy.fetch(vh, v_row_stride, (t + 1) * kFwdBlockN, p.Skv, tid);
+    }
+
+    if (t < n_tiles_wave) {
+      // ---- S^T = K Q^T : [64 keys] x [64 queries] as 2 x 2 tiles of 32 x 32
+      f32x16 s[2][2];
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) s[kvb][qb][v] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb) {
+          const bf16x8 a = lds_read_straight(ktile, KP, kvb * 32 + c, ks * 16 + g * 8);
+          s[kvb][0] = mfma32(a, qf[0][ks], s[kvb][0]);
+          s[kvb][1] = mfma32(a, qf[1][ks], s[kvb][1]);
+        }
+      }
+
+      // ---- mask (diagonal tile of a causal chunk, or a ragged last tile)
+      const int n0 = t * kFwdBlockN;
+      const bool diag = CAUSAL && (t == n_tiles_wave - 1) && (n0 + kFwdBlockN - 1 > q_wave0);
+      const bool ragged = n0 + kFwdBlockN > p.Skv;
+      if (diag || ragged) {
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          const int qrow = q_wave0 + qb * 32 + c;
+          const int limit = CAUSAL ? min(qrow, p.Skv - 1) : p.Skv - 1;  // last visible key
+#pragma unroll
+          for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int key = n0 + kvb * 32 + acc_row(v, g);
+              if (key > limit) s[kvb][qb][v] = -INFINITY;
+            }
+        }
+      }
+
+      // ---- online softmax, one query column per lane pair
+      bf16x8 pf[2][4];  // P^T as B operand: [query block][contraction step of 16 keys]
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        float mx = s[0][qb][0];
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kvb][qb][v]);
+        mx = pair_max(mx);
+        const float m_new = fmaxf(m_run[qb], mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row with no visible key yet
+        const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_use) * p.kappa);
+        const float mk = m_use * p.kappa;
+        m_run[qb] = m_new;
+        float rs = 0.f;
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const float e = __builtin_amdgcn_exp2f(s[kvb][qb][v] * p.kappa - mk);
+            s[kvb][qb][v] = e;
+            rs += e;
+          }
+        l_run[qb] = l_run[qb] * alpha + rs;
+#pragma unroll
+        for (int i = 0; i < DVB; ++i)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) oacc[i][qb][v] *= alpha;
+#pragma unroll
+        for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            const f32x16& x = s[kvb][qb];
+            pf[qb][2 * kvb + jj] = to_bf16x8(x[8 * jj], x[8 * jj + 1], x[8 * jj + 2], x[8 * jj + 3], x[8 * jj + 4],
+                                             x[8 * jj + 5], x[8 * jj + 6], x[8 * jj + 7]);
+          }
+      }
+
+      // ---- O^T += V^T P^T
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int i = 0; i < DVB; ++i) {
+          const bf16x8 a = lds_read_transposed(vtile, VP, 16 * j, 32 * i, lane);
+          oacc[i][0] = mfma32(a, pf[0][j], oacc[i][0]);
+          oacc[i][1] = mfma32(a, pf[1][j], oacc[i][1]);
+        }
+      }
+    }
+
+    if (have_next) {
+      char* nk = smem + ((t + 1) & 1) * (kKTile + kVTile);
+      kcopy.commit(nk, tid);
+      vcopy.commit(nk + kKTile, tid);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: normalise, store O (bf16) and LSE2
+  __bf16* oh = p.o + b * p.o_bs + (int64_t)h * DV;
+  float* lse = p.lse + b * p.lse_bs + (int64_t)h * p.lse_hs;
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qrow = q_wave0 + qb * 32 + c;
+    const float l = pair_sum(l_run[qb]);
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    if (qrow < p.Sq) {
+      __bf16* dst = oh + qrow * o_row_stride;
+#pragma unroll
+      for (int i = 0; i < DVB; ++i)
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          u32x2 w;
+          w[0] = pack_bf16x2(oacc[i][qb][4 * b4] * inv, oacc[i][qb][4 * b4 + 1] * inv);
+          w[1] = pack_bf16x2(oacc[i][qb][4 * b4 + 2] * inv, oacc[i][qb][4 * b4 + 3] * inv);
+          *reinterpret_cast<u32x2*>(dst + 32 * i + 8 * b4 + 4 * g) = w;
+        }
+      if (g == 0) lse[qrow] = (l > 0.f) ? __builtin_amdgcn_logf(l) + m_run[qb] * p.kappa : -INFINITY;
+    }
+  }
+}
+
+template <int DQK, int DV>
+void launch_fwd(const FwdParams& p, bool causal, dim3 grid, hipStream_t st) {
+  if (causal)
+    hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV, true>), grid, dim3(kFwdThreads), 0, st, p);
+  else
+    hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV, false>), grid, dim3(kFwdThreads), 0, st, p);
+}
+
+}  // namespace
+}  // namespace pith
+
+using namespace pith;
+
+extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) {
+  if (!a) return fail(PITH_ERR_NULL_POINTER, "pith_attn_fwd: args is NULL");
+  if (!a->q || !a->k || !a->v || !a->o || !a->lse) return fail(PITH_ERR_NULL_POINTER, "pith_attn_fwd: NULL tensor pointer");
+  if (a->B <= 0 || a->Sq <= 0 || a->Skv <= 0 || a->Hq <= 0 || a->Hkv <= 0)
+    return fail(PITH_ERR_BAD_SHAPE, "pith_attn_fwd: B=%lld Sq=%lld Skv=%lld Hq=%lld Hkv=%lld must all be positive",
+                (long long)a->B, (long long)a->Sq, (long long)a->Skv, (long long)a->Hq, (long long)a->Hkv);
+  if (a->Hq % a->Hkv != 0)
+    return fail(PITH_ERR_BAD_SHAPE, "pith_attn_fwd: Hq=%lld is not a multiple of Hkv=%lld", (long long)a->Hq,
+                (long long)a->Hkv);
+  if (a->causal && a->Sq != a->Skv)
+    return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: causal needs Sq == Skv (got %lld, %lld)", (long long)a->Sq,
+                (long long)a->Skv);
+  if (a->Sq > (1 << 24) || a->Skv > (1 << 24) || a->Hq > 65535 || a->B > 65535)
+    return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: sequence, head or batch count beyond the launch grid limits");
+  if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->o) || a->q_bs % 8 || a->k_bs % 8 ||
+      a->v_bs % 8 || a->o_bs % 8)
+    return fail(PITH_ERR_MISALIGNED, "pith_attn_fwd: tensor pointers / batch strides must keep 16-byte alignment");
+
+  FwdParams p;
+  p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v;
+  p.o = (__bf16*)a->o; p.lse = a->lse;
+  p.Sq = (int)a->Sq; p.Skv = (int)a->Skv; p.Hq = (int)a->Hq; p.Hkv = (int)a->Hkv; p.group = (int)(a->Hq / a->Hkv);
+  p.m_tiles = (int)((a->Sq + kFwdBlockM - 1) / kFwdBlockM);
+  p.q_bs = a->q_bs; p.k_bs = a->k_bs; p.v_bs = a->v_bs; p.o_bs = a->o_bs; p.lse_bs = a->lse_bs; p.lse_hs = a->lse_hs;
+  p.kappa = a->scale * 1.44269504088896340736f;
+  const dim3 grid((unsigned)p.m_tiles, (unsigned)a->Hq, (unsigned)a->B);
+  hipStream_t st = (hipStream_t)stream;
+  if (a->Dqk == 128 && a->Dv == 128) launch_fwd<128, 128>(p, a->causal != 0, grid, st);
+  else if (a->Dqk == 192 && a->Dv == 128) launch_fwd<192, 128>(p, a->causal != 0, grid, st);
+  else if (a->Dqk == 64 && a->Dv == 64) launch_fwd<64, 64>(p, a->causal != 0, grid, st);
+  else
+    return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: head dims (Dqk=%lld, Dv=%lld) not in {(64,64),(128,128),(192,128)}",
+                (long long)a->Dqk, (long long)a->Dv);
+  return check_launch("pith_attn_fwd");
+}

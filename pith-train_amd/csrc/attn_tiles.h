@@ -1,0 +1,116 @@
+// Device building blocks shared by the attention kernels (forward, dQ, dK/dV) on gfx950.
+//
+// Matrix-core conventions used everywhere (v_mfma_f32_32x32x16_bf16, one wavefront of 64 lanes,
+// lane = 32*g + c with c = lane % 32, g = lane / 32):
+//   A operand (32 x 16): lane holds row c, contraction slots k = 8*g + e, e = 0..7
+//   B operand (16 x 32): lane holds column c, the same contraction slots
+//   C/D      (32 x 32): lane holds column c, rows 8*(v/4) + 4*g + v%4, v = 0..15
+// A result tile can therefore be fed back as the B operand of a product that contracts over
+// its ROW index without leaving registers: slot (g, e) of contraction step j then stands for
+// row 16*j + 8*(e/4) + 4*g + e%4 of the tile ("slot order"). The other operand of that product
+// is fetched from LDS in the same slot order.
+//
+// Tiles streamed through LDS are row-major [row][col] bf16 with a padded pitch. They are read
+//   - "straight": lane takes 8 consecutive columns of row c            (one ds_read_b128), or
+//   - "transposed": lane takes column c at 8 rows in slot order         (two ds_read_b64_tr_b16).
+#pragma once
+
+#include "pith_common.h"
+
+namespace pith {
+
+typedef __attribute__((address_space(3))) char lds_char;
+
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// Straight A/B fragment: row `row`, columns col0 .. col0+7 (col0 multiple of 8).
+__device__ __forceinline__ bf16x8 lds_read_straight(const char* tile, int pitch, int row, int col0) {
+  return *reinterpret_cast<const bf16x8*>(tile + row * pitch + col0 * 2);
+}
+
+// Transposed fragment in slot order. For a wavefront the result is the A (or B) operand whose
+// non-contracted index is the tile COLUMN col_base + c and whose contraction slots (g, e) are
+// the tile ROWS row_base + 8*(e/4) + 4*g + e%4.
+// ds_read_b64_tr_b16 works on blocks of 16 lanes: lane r of a block supplies the address of 4
+// consecutive columns; lanes 4i..4i+3 of the block must cover 16 consecutive columns of row i;
+// lane r then receives column r of rows 0..3 of the block.
+__device__ __forceinline__ bf16x8 lds_read_transposed(const char* tile, int pitch, int row_base, int col_base,
+                                                      int lane) {
+  const int r = lane & 15, blk = lane >> 4;
+  const int row = row_base + 4 * (blk >> 1) + (r >> 2);
+  const int col = col_base + 16 * (blk & 1) + 4 * (r & 3);
+  const char* p = tile + row * pitch + col * 2;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 8 * pitch));
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  s16x8 v;
+  v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
+  v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// Row index (0..31) inside a 32x32 result tile of accumulator element v for lane group g.
+__device__ __forceinline__ int acc_row(int v, int g) { return 8 * (v >> 2) + 4 * g + (v & 3); }
+
+// max / sum across the two lanes (c, c+32) that share a result column.
+__device__ __forceinline__ float pair_max(float x) {
+  const int xi = __float_as_int(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+  return fmaxf(__int_as_float(r[0]), __int_as_float(r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  const int xi = __float_as_int(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+  return __int_as_float(r[0]) + __int_as_float(r[1]);
+}
+
+// Eight fp32 accumulator values -> bf16 fragment (round-to-nearest-even).
+__device__ __forceinline__ bf16x8 to_bf16x8(float a0, float a1, float a2, float a3, float a4, float a5, float a6,
+                                            float a7) {
+  bf16x8 r;
+  r[0] = (__bf16)a0; r[1] = (__bf16)a1; r[2] = (__bf16)a2; r[3] = (__bf16)a3;
+  r[4] = (__bf16)a4; r[5] = (__bf16)a5; r[6] = (__bf16)a6; r[7] = (__bf16)a7;
+  return r;
+}
+
+// Cooperative copy of a [ROWS x COLS] bf16 tile between global memory and LDS by THREADS threads,
+// split into a "fetch to registers" half and a "store to LDS" half so that the global loads of
+// the next tile can be in flight while the current tile is consumed.
+template <int ROWS, int COLS, int PITCH, int THREADS>
+struct TileCopy {
+  static constexpr int kChunksPerRow = COLS / 8;
+  static constexpr int kChunks = ROWS * kChunksPerRow;
+  static constexpr int kPerThread = (kChunks + THREADS - 1) / THREADS;
+  u32x4 regs[kPerThread];
+
+  // src: address of element [row 0][col 0] of the tile's head slice; row_stride in elements;
+  // rows at or beyond `valid_rows` are read from the last valid row (their values are masked
+  // or discarded by the caller).
+  __device__ __forceinline__ void fetch(const __bf16* src, int64_t row_stride, int row0, int valid_rows, int tid) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      const int c = tid + i * THREADS;
+      if (kChunks % THREADS == 0 || c < kChunks) {
+        const int row = c / kChunksPerRow, col = c - row * kChunksPerRow;
+        int grow = row0 + row;
+        grow = grow < valid_rows ? grow : valid_rows - 1;
+        regs[i] = *reinterpret_cast<const u32x4*>(src + grow * row_stride + col * 8);
+      }
+    }
+  }
+  __device__ __forceinline__ void commit(char* tile, int tid) const {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      const int c = tid + i * THREADS;
+      if (kChunks % THREADS == 0 || c < kChunks) {
+        const int row = c / kChunksPerRow, col = c - row * kChunksPerRow;
+        *reinterpret_cast<u32x4*>(tile + row * PITCH + col * 16) = regs[i];
+      }
+    }
+  }
+};
+
+}  // namespace pith

@@ -1,0 +1,313 @@
+// Online-softmax combine of two partial attention results, plus the two small streaming
+// kernels of the path (delta = rowsum(O*dO), fp32 -> bf16 cast). All three are HBM-bound:
+// every byte of the operands is read once and every byte of the result written once, with
+// 16-byte accesses that are contiguous across a wavefront.
+//
+// Combine follows pithtrain/operators/ring_attention/mla.py:27-40 (base 2) and
+// pithtrain/operators/ring_attention/standard.py:53-66 (base e).
+#include "pith_common.h"
+
+namespace pith {
+namespace {
+
+constexpr int kCombineThreads = 256;
+
+// 8 consecutive elements of a bf16 or fp32 row.
+template <typename T>
+struct Vec8;
+
+template <>
+struct Vec8<__bf16> {
+  u32x4 raw;
+  __device__ __forceinline__ void load(const __bf16* p) { raw = *reinterpret_cast<const u32x4*>(p); }
+  __device__ __forceinline__ void store(__bf16* p) const { *reinterpret_cast<u32x4*>(p) = raw; }
+  __device__ __forceinline__ float get(int i) const {
+    uint32_t w = raw[i >> 1];
+    return (i & 1) ? bf16hi_to_f32(w) : bf16lo_to_f32(w);
+  }
+  __device__ __forceinline__ void set_pair(int pair, float a, float b) { raw[pair] = pack_bf16x2(a, b); }
+};
+
+template <>
+struct Vec8<float> {
+  f32x4 lo, hi;
+  __device__ __forceinline__ void load(const float* p) {
+    lo = *reinterpret_cast<const f32x4*>(p);
+    hi = *reinterpret_cast<const f32x4*>(p + 4);
+  }
+  __device__ __forceinline__ void store(float* p) const {
+    *reinterpret_cast<f32x4*>(p) = lo;
+    *reinterpret_cast<f32x4*>(p + 4) = hi;
+  }
+  __device__ __forceinline__ float get(int i) const { return i < 4 ? lo[i] : hi[i - 4]; }
+  __device__ __forceinline__ void set_pair(int pair, float a, float b) {
+    if (pair < 2) {
+      lo[2 * pair] = a;
+      lo[2 * pair + 1] = b;
+    } else {
+      hi[2 * pair - 4] = a;
+      hi[2 * pair - 3] = b;
+    }
+  }
+};
+
+struct CombineParams {
+  const void* out1;
+  const float* lse1;
+  const void* out2;
+  const float* lse2;
+  void* out;
+  float* lse_out;
+  int64_t S;
+  int H, D8;  // D8 = D / 8 chunks of 16 bytes (bf16) per head row
+  int tile_s;
+  int base_e;
+  int64_t out1_bs, out2_bs, out_bs;
+  int64_t lse1_bs, lse1_hs, lse2_bs, lse2_hs, lse_out_bs, lse_out_hs;
+};
+
+// One block = `tile_s` consecutive sequence positions of one batch element, all heads.
+// Stage 1: the [H, tile_s] patch of both LSE tensors is read (contiguous along s), the two
+//          normalised weights are left in LDS and the merged LSE is written.
+// Stage 2: the [tile_s, H, D] slab of O, which is one contiguous range of memory, is streamed
+//          with 16-byte accesses; thread t owns chunks t, t+256, ...
+template <typename T1, typename T2, typename TO>
+__global__ __launch_bounds__(kCombineThreads) void combine_kernel(CombineParams p) {
+  extern __shared__ float weights[];  // [rows][2], rows = tile_s * H, row = s_local * H + h
+  const int b = blockIdx.y;
+  const int64_t s0 = (int64_t)blockIdx.x * p.tile_s;
+  const int ts = (int)min((int64_t)p.tile_s, p.S - s0);
+  const int rows = ts * p.H;
+
+  const float* l1 = p.lse1 + b * p.lse1_bs + s0;
+  const float* l2 = p.lse2 + b * p.lse2_bs + s0;
+  float* lo = p.lse_out + b * p.lse_out_bs + s0;
+  for (int i = threadIdx.x; i < rows; i += kCombineThreads) {
+    const int h = i / ts, sl = i - h * ts;
+    const float a = l1[h * p.lse1_hs + sl];
+    const float c = l2[h * p.lse2_hs + sl];
+    const float m = fmaxf(a, c);
+    float w1, w2, lse;
+    if (m == -INFINITY) {
+      // Both partials are empty: the reference yields NaN here (-inf - -inf); an empty
+      // result (weights 0, lse -inf) is returned instead. The ring never produces this case.
+      w1 = 0.f;
+      w2 = 0.f;
+      lse = -INFINITY;
+    } else {
+      float e1, e2;
+      if (p.base_e) {
+        e1 = expf(a - m);
+        e2 = expf(c - m);
+      } else {
+        e1 = exp2f(a - m);
+        e2 = exp2f(c - m);
+      }
+      const float sum = e1 + e2;
+      w1 = e1 / sum;
+      w2 = e2 / sum;
+      lse = m + (p.base_e ? logf(sum) : log2f(sum));
+    }
+    weights[2 * (sl * p.H + h)] = w1;
+    weights[2 * (sl * p.H + h) + 1] = w2;
+    lo[h * p.lse_out_hs + sl] = lse;
+  }
+  __syncthreads();
+
+  const int64_t slab = (s0 * p.H) * (int64_t)p.D8 * 8;
+  const T1* o1 = reinterpret_cast<const T1*>(p.out1) + b * p.out1_bs + slab;
+  const T2* o2 = reinterpret_cast<const T2*>(p.out2) + b * p.out2_bs + slab;
+  TO* oo = reinterpret_cast<TO*>(p.out) + b * p.out_bs + slab;
+  const int chunks = rows * p.D8;
+
+  constexpr int kUnroll = 4;
+  for (int c0 = threadIdx.x; c0 < chunks; c0 += kCombineThreads * kUnroll) {
+    Vec8<T1> x[kUnroll];
+    Vec8<T2> y[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int c = c0 + u * kCombineThreads;
+      if (c < chunks) {
+        x[u].load(o1 + (int64_t)c * 8);
+        y[u].load(o2 + (int64_t)c * 8);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int c = c0 + u * kCombineThreads;
+      if (c < chunks) {
+        const int row = c / p.D8;
+        const float w1 = weights[2 * row], w2 = weights[2 * row + 1];
+        Vec8<TO> r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float v0 = w1 * x[u].get(2 * j) + w2 * y[u].get(2 * j);
+          const float v1 = w1 * x[u].get(2 * j + 1) + w2 * y[u].get(2 * j + 1);
+          r.set_pair(j, v0, v1);
+        }
+        r.store(oo + (int64_t)c * 8);
+      }
+    }
+  }
+}
+
+template <typename T1, typename T2>
+void launch_combine_t2(const CombineParams& p, int dtype_out, dim3 grid, size_t lds, hipStream_t st) {
+  if (dtype_out == PITH_BF16)
+    hipLaunchKernelGGL((combine_kernel<T1, T2, __bf16>), grid, dim3(kCombineThreads), lds, st, p);
+  else
+    hipLaunchKernelGGL((combine_kernel<T1, T2, float>), grid, dim3(kCombineThreads), lds, st, p);
+}
+
+// ---------------------------------------------------------------------------------------------
+// delta[b,h,s] = sum_d O*dO (pithtrain/operators/mla/triton.py:101-122). One block handles
+// `tile_s` consecutive positions x all heads; the [tile_s, H, D] slabs of O and dO are contiguous.
+// D/8 consecutive lanes own one (s,h) row and reduce with DPP-free shuffles; the per-row sums go
+// through LDS so the [H, tile_s] patch of delta is written contiguously along s.
+struct DeltaParams {
+  const __bf16* o;
+  const __bf16* dout;
+  float* delta;
+  int64_t S;
+  int H, D8, tile_s;
+  int64_t o_bs, dout_bs, delta_bs, delta_hs;
+};
+
+constexpr int kDeltaThreads = 256;
+
+__global__ __launch_bounds__(kDeltaThreads) void delta_kernel(DeltaParams p) {
+  extern __shared__ float rowsum[];  // [tile_s * H]
+  const int b = blockIdx.y;
+  const int64_t s0 = (int64_t)blockIdx.x * p.tile_s;
+  const int ts = (int)min((int64_t)p.tile_s, p.S - s0);
+  const int rows = ts * p.H;
+  const int64_t slab = (s0 * p.H) * (int64_t)p.D8 * 8;
+  const __bf16* o = p.o + b * p.o_bs + slab;
+  const __bf16* g = p.dout + b * p.dout_bs + slab;
+  const int chunks = rows * p.D8;
+  // D8 is a power of two <= 64 (checked on the host), so the lanes of one row sit inside one wave.
+  for (int c0 = 0; c0 < chunks; c0 += kDeltaThreads) {
+    const int c = c0 + threadIdx.x;
+    float acc = 0.f;
+    if (c < chunks) {
+      Vec8<__bf16> x, y;
+      x.load(o + (int64_t)c * 8);
+      y.load(g + (int64_t)c * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc += x.get(j) * y.get(j);
+    }
+    for (int off = p.D8 >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    if (c < chunks && (c & (p.D8 - 1)) == 0) rowsum[c / p.D8] = acc;
+  }
+  __syncthreads();
+  float* d = p.delta + b * p.delta_bs + s0;
+  for (int i = threadIdx.x; i < rows; i += kDeltaThreads) {
+    const int h = i / ts, sl = i - h * ts;
+    d[h * p.delta_hs + sl] = rowsum[sl * p.H + h];
+  }
+}
+
+__global__ __launch_bounds__(256) void cast_f32_bf16_kernel(const float* __restrict__ src, __bf16* __restrict__ dst,
+                                                            int64_t n8) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += (int64_t)gridDim.x * blockDim.x) {
+    Vec8<float> x;
+    x.load(src + i * 8);
+    Vec8<__bf16> y;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) y.set_pair(j, x.get(2 * j), x.get(2 * j + 1));
+    y.store(dst + i * 8);
+  }
+}
+
+// Rows per block: as many as keep the grid at several blocks per CU and the LDS patch small.
+int pick_tile_s(int64_t B, int64_t S, int64_t H, int max_rows) {
+  int ts = 16;
+  while (ts > 1 && (B * ((S + ts - 1) / ts) < 2048 || ts * H > max_rows)) ts >>= 1;
+  return ts;
+}
+
+}  // namespace
+}  // namespace pith
+
+using namespace pith;
+
+extern "C" int pith_combine(const pith_combine_args* a, pith_stream_t stream) {
+  if (!a) return fail(PITH_ERR_NULL_POINTER, "pith_combine: args is NULL");
+  if (!a->out1 || !a->lse1 || !a->out2 || !a->lse2 || !a->out || !a->lse_out)
+    return fail(PITH_ERR_NULL_POINTER, "pith_combine: NULL tensor pointer");
+  if (a->B <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0)
+    return fail(PITH_ERR_BAD_SHAPE, "pith_combine: B=%lld S=%lld H=%lld D=%lld must all be positive", (long long)a->B,
+                (long long)a->S, (long long)a->H, (long long)a->D);
+  if (a->D % 8 != 0) return fail(PITH_ERR_BAD_SHAPE, "pith_combine: D=%lld is not a multiple of 8", (long long)a->D);
+  if (a->H > 4096 || a->B > 65535)
+    return fail(PITH_ERR_UNSUPPORTED, "pith_combine: H=%lld > 4096 or B=%lld > 65535", (long long)a->H,
+                (long long)a->B);
+  const int dts[3] = {a->dtype1, a->dtype2, a->dtype_out};
+  for (int dt : dts)
+    if (dt != PITH_BF16 && dt != PITH_F32) return fail(PITH_ERR_BAD_DTYPE, "pith_combine: dtype %d is not bf16/fp32", dt);
+  if (a->base != PITH_BASE_2 && a->base != PITH_BASE_E)
+    return fail(PITH_ERR_BAD_DTYPE, "pith_combine: base %d is not PITH_BASE_2/PITH_BASE_E", a->base);
+  if (!aligned16(a->out1) || !aligned16(a->out2) || !aligned16(a->out) || a->out1_bs % 8 || a->out2_bs % 8 ||
+      a->out_bs % 8)
+    return fail(PITH_ERR_MISALIGNED, "pith_combine: O pointers / batch strides must keep 16-byte alignment");
+  const int64_t slab = a->S * a->H * a->D;
+  if (a->B > 1 && (a->out1_bs < slab || a->out2_bs < slab || a->out_bs < slab))
+    return fail(PITH_ERR_BAD_SHAPE, "pith_combine: an O batch stride is smaller than S*H*D");
+
+  CombineParams p;
+  p.out1 = a->out1; p.lse1 = a->lse1; p.out2 = a->out2; p.lse2 = a->lse2; p.out = a->out; p.lse_out = a->lse_out;
+  p.S = a->S; p.H = (int)a->H; p.D8 = (int)(a->D / 8);
+  p.base_e = a->base == PITH_BASE_E;
+  p.out1_bs = a->out1_bs; p.out2_bs = a->out2_bs; p.out_bs = a->out_bs;
+  p.lse1_bs = a->lse1_bs; p.lse1_hs = a->lse1_hs; p.lse2_bs = a->lse2_bs; p.lse2_hs = a->lse2_hs;
+  p.lse_out_bs = a->lse_out_bs; p.lse_out_hs = a->lse_out_hs;
+  p.tile_s = pick_tile_s(a->B, a->S, a->H, 4096);
+  const dim3 grid((unsigned)((a->S + p.tile_s - 1) / p.tile_s), (unsigned)a->B);
+  const size_t lds = (size_t)p.tile_s * p.H * 2 * sizeof(float);
+  hipStream_t st = (hipStream_t)stream;
+  if (a->dtype1 == PITH_BF16) {
+    if (a->dtype2 == PITH_BF16) launch_combine_t2<__bf16, __bf16>(p, a->dtype_out, grid, lds, st);
+    else launch_combine_t2<__bf16, float>(p, a->dtype_out, grid, lds, st);
+  } else {
+    if (a->dtype2 == PITH_BF16) launch_combine_t2<float, __bf16>(p, a->dtype_out, grid, lds, st);
+    else launch_combine_t2<float, float>(p, a->dtype_out, grid, lds, st);
+  }
+  return check_launch("pith_combine");
+}
+
+extern "C" int pith_attn_bwd_delta(const pith_attn_delta_args* a, pith_stream_t stream) {
+  if (!a) return fail(PITH_ERR_NULL_POINTER, "pith_attn_bwd_delta: args is NULL");
+  if (!a->o || !a->dout || !a->delta) return fail(PITH_ERR_NULL_POINTER, "pith_attn_bwd_delta: NULL tensor pointer");
+  if (a->B <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0)
+    return fail(PITH_ERR_BAD_SHAPE, "pith_attn_bwd_delta: B=%lld S=%lld H=%lld D=%lld must all be positive",
+                (long long)a->B, (long long)a->S, (long long)a->H, (long long)a->D);
+  const int64_t d8 = a->D / 8;
+  if (a->D % 8 != 0 || d8 > 64 || (d8 & (d8 - 1)) != 0)
+    return fail(PITH_ERR_UNSUPPORTED, "pith_attn_bwd_delta: D=%lld must be 8 * a power of two, at most 512",
+                (long long)a->D);
+  if (a->H > 4096 || a->B > 65535)
+    return fail(PITH_ERR_UNSUPPORTED, "pith_attn_bwd_delta: H=%lld > 4096 or B=%lld > 65535", (long long)a->H,
+                (long long)a->B);
+  if (!aligned16(a->o) || !aligned16(a->dout) || a->o_bs % 8 || a->dout_bs % 8)
+    return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_delta: O/dO pointers / batch strides must keep 16-byte alignment");
+  DeltaParams p;
+  p.o = (const __bf16*)a->o; p.dout = (const __bf16*)a->dout; p.delta = a->delta;
+  p.S = a->S; p.H = (int)a->H; p.D8 = (int)d8;
+  p.o_bs = a->o_bs; p.dout_bs = a->dout_bs; p.delta_bs = a->delta_bs; p.delta_hs = a->delta_hs;
+  p.tile_s = pick_tile_s(a->B, a->S, a->H, 8192);
+  const dim3 grid((unsigned)((a->S + p.tile_s - 1) / p.tile_s), (unsigned)a->B);
+  hipLaunchKernelGGL(delta_kernel, grid, dim3(kDeltaThreads), (size_t)p.tile_s * p.H * sizeof(float),
+                     (hipStream_t)stream, p);
+  return check_launch("pith_attn_bwd_delta");
+}
+
+extern "C" int pith_cast_f32_bf16(const float* src, void* dst, int64_t n, pith_stream_t stream) {
+  if (!src || !dst) return fail(PITH_ERR_NULL_POINTER, "pith_cast_f32_bf16: NULL pointer");
+  if (n <= 0 || n % 8 != 0) return fail(PITH_ERR_BAD_SHAPE, "pith_cast_f32_bf16: n=%lld must be a positive multiple of 8", (long long)n);
+  if (!aligned16(src) || !aligned16(dst)) return fail(PITH_ERR_MISALIGNED, "pith_cast_f32_bf16: pointers must be 16-byte aligned");
+  const int64_t n8 = n / 8;
+  const int64_t blocks = (n8 + 255) / 256;
+  hipLaunchKernelGGL(cast_f32_bf16_kernel, dim3((unsigned)(blocks < 16384 ? blocks : 16384)), dim3(256), 0,
+                     (hipStream_t)stream, src, (__bf16*)dst, n8);
+  return check_launch("pith_cast_f32_bf16");
+}

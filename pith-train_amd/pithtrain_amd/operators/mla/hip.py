@@ -1,0 +1,223 @@
+"""
+Per-chunk attention operators backed by libpith_hip.so (HIP kernels for gfx950).
+
+Drop-in for the raw helpers of pithtrain/operators/mla/triton.py:552-603 (same names, argument
+order and return values), generalised beyond the reference's dq=192/dv=128 MHA case to what the
+ring needs on both model families:
+
+  * head dims (Dqk, Dv) in {(64, 64), (128, 128), (192, 128)};
+  * grouped-query attention (k/v with fewer heads than q; dk/dv sum over the group);
+  * non-causal calls with different query and key lengths (zigzag half-chunk steps);
+  * arguments that are slices along S of contiguous tensors (no copies are made).
+
+ b : batch size, s : sequence length, h : heads, dq : query/key head dim, dv : value head dim.
+Layouts: q/k/v/o/do/dq/dk/dv are BSHD bf16; lse and delta are [b, h, s] fp32; lse is base-2.
+
+The `*_into` functions write into caller-provided tensors and are what the ring drivers use;
+the underscore helpers allocate their outputs like the reference does.
+"""
+
+import math
+
+import torch
+import torch.nn as nn
+
+from pithtrain_amd import _C
+
+SUPPORTED_HEAD_DIMS = ((64, 64), (128, 128), (192, 128))
+
+
+def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool) -> None:
+    _C.require_device(q, k, v)
+    assert q.dtype == k.dtype == v.dtype == torch.bfloat16, "q, k, v must be bfloat16"
+    assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be [B, S, H, D]"
+    d_q, d_v = q.shape[-1], v.shape[-1]
+    assert (d_q, d_v) in SUPPORTED_HEAD_DIMS, (
+        f"HIP attention kernels support (dq, dv) in {SUPPORTED_HEAD_DIMS}, got dq={d_q} and dv={d_v}"
+    )
+    assert k.shape[-1] == d_q, f"k head dim {k.shape[-1]} != q head dim {d_q}"
+    assert k.shape[0] == q.shape[0] and v.shape[0] == q.shape[0], "batch sizes differ"
+    assert k.shape[1] == v.shape[1] and k.shape[2] == v.shape[2], "k and v disagree on sequence length or heads"
+    assert q.shape[2] % k.shape[2] == 0, f"q heads {q.shape[2]} not a multiple of kv heads {k.shape[2]}"
+    if causal:
+        assert q.shape[1] == k.shape[1], "causal attention needs equal query and key lengths"
+
+
+def attn_fwd_into(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
+    softmax_scale: float, causal: bool,
+) -> None:  # fmt: skip
+    """o, lse <- attention(q, k, v). o [b, sq, hq, dv] bf16 and lse [b, hq, sq] fp32 are written."""
+    _check_qkv(q, k, v, causal)
+    _C.require_device(q, o, lse)
+    b, sq, hq, d_q = q.shape
+    _, skv, hkv, d_v = v.shape
+    assert o.dtype == torch.bfloat16 and tuple(o.shape) == (b, sq, hq, d_v), "o has the wrong dtype or shape"
+    assert lse.dtype == torch.float32 and tuple(lse.shape) == (b, hq, sq), "lse has the wrong dtype or shape"
+    lse_bs, lse_hs = _C.bhs_strides(lse, "lse")
+    args = _C.AttnFwdArgs(
+        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), o=o.data_ptr(), lse=lse.data_ptr(),
+        B=b, Sq=sq, Skv=skv, Hq=hq, Hkv=hkv, Dqk=d_q, Dv=d_v,
+        q_bs=_C.bshd_batch_stride(q, "q"), k_bs=_C.bshd_batch_stride(k, "k"),
+        v_bs=_C.bshd_batch_stride(v, "v"), o_bs=_C.bshd_batch_stride(o, "o"),
+        lse_bs=lse_bs, lse_hs=lse_hs, scale=float(softmax_scale), causal=int(bool(causal)),
+    )  # fmt: skip
+    _C.check(_C.lib().pith_attn_fwd(_C.byref(args), _C.current_stream(q)))
+
+
+def attn_bwd_delta_into(out: torch.Tensor, dout: torch.Tensor, delta: torch.Tensor) -> None:
+    """delta[b, h, s] <- sum_d out * dout (fp32)."""
+    _C.require_device(out, dout, delta)
+    assert out.dtype == dout.dtype == torch.bfloat16 and out.shape == dout.shape, "out/dout mismatch"
+    b, s, h, d_v = out.shape
+    assert delta.dtype == torch.float32 and tuple(delta.shape) == (b, h, s), "delta has the wrong dtype or shape"
+    d_bs, d_hs = _C.bhs_strides(delta, "delta")
+    args = _C.AttnDeltaArgs(
+        o=out.data_ptr(), dout=dout.data_ptr(), delta=delta.data_ptr(), B=b, S=s, H=h, D=d_v,
+        o_bs=_C.bshd_batch_stride(out, "out"), dout_bs=_C.bshd_batch_stride(dout, "dout"),
+        delta_bs=d_bs, delta_hs=d_hs,
+    )  # fmt: skip
+    _C.check(_C.lib().pith_attn_bwd_delta(_C.byref(args), _C.current_stream(out)))
+
+
+def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal) -> _C.AttnBwdArgs:
+    _check_qkv(q, k, v, causal)
+    _C.require_device(q, dout, lse, delta)
+    b, sq, hq, d_q = q.shape
+    _, skv, hkv, d_v = v.shape
+    assert dout.dtype == torch.bfloat16 and tuple(dout.shape) == (b, sq, hq, d_v), "dout has the wrong dtype or shape"
+    for name, t in (("lse", lse), ("delta", delta)):
+        assert t.dtype == torch.float32 and tuple(t.shape) == (b, hq, sq), f"{name} has the wrong dtype or shape"
+    lse_bs, lse_hs = _C.bhs_strides(lse, "lse")
+    assert _C.bhs_strides(delta, "delta") == (lse_bs, lse_hs), "lse and delta must share strides"
+    return _C.AttnBwdArgs(
+        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), dout=dout.data_ptr(),
+        lse=lse.data_ptr(), delta=delta.data_ptr(), dq=None, dk=None, dv=None,
+        B=b, Sq=sq, Skv=skv, Hq=hq, Hkv=hkv, Dqk=d_q, Dv=d_v,
+        q_bs=_C.bshd_batch_stride(q, "q"), k_bs=_C.bshd_batch_stride(k, "k"),
+        v_bs=_C.bshd_batch_stride(v, "v"), dout_bs=_C.bshd_batch_stride(dout, "dout"),
+        dq_bs=0, dk_bs=0, dv_bs=0, lse_bs=lse_bs, lse_hs=lse_hs,
+        scale=float(softmax_scale), causal=int(bool(causal)),
+        dq_dtype=_C.PITH_BF16, dkv_dtype=_C.PITH_BF16, accumulate_dq=0, accumulate_dkv=0,
+    )  # fmt: skip
+
+
+def attn_bwd_dkdv_into(
+    q, k, v, dout, lse, delta, dk: torch.Tensor, dv: torch.Tensor, softmax_scale: float, causal: bool,
+    accumulate: bool = False,
+) -> None:  # fmt: skip
+    """dk, dv <- (or +=, with accumulate) the gradients of this chunk pair; bf16 or fp32 outputs."""
+    args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal)
+    _C.require_device(q, dk, dv)
+    assert dk.shape == k.shape and dv.shape == v.shape and dk.dtype == dv.dtype, "dk/dv must match k/v"
+    args.dk, args.dv = dk.data_ptr(), dv.data_ptr()
+    args.dk_bs, args.dv_bs = _C.bshd_batch_stride(dk, "dk"), _C.bshd_batch_stride(dv, "dv")
+    args.dkv_dtype = _C.dtype_code(dk)
+    args.accumulate_dkv = int(bool(accumulate))
+    _C.check(_C.lib().pith_attn_bwd_dkdv(_C.byref(args), _C.current_stream(q)))
+
+
+def attn_bwd_dq_into(
+    q, k, v, dout, lse, delta, dq: torch.Tensor, softmax_scale: float, causal: bool, accumulate: bool = False,
+) -> None:  # fmt: skip
+    """dq <- (or +=, with accumulate) the query gradient of this chunk pair; bf16 or fp32 output."""
+    args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal)
+    _C.require_device(q, dq)
+    assert dq.shape == q.shape, "dq must match q"
+    args.dq = dq.data_ptr()
+    args.dq_bs = _C.bshd_batch_stride(dq, "dq")
+    args.dq_dtype = _C.dtype_code(dq)
+    args.accumulate_dq = int(bool(accumulate))
+    _C.check(_C.lib().pith_attn_bwd_dq(_C.byref(args), _C.current_stream(q)))
+
+
+# ---------------------------------------------------------------------------------------------
+# Reference-named helpers (pithtrain/operators/mla/triton.py:552-603)
+
+
+def _mla_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float, causal: bool = True):
+    """Raw attention forward. Returns (out, lse) with lse in log2 scale."""
+    (b, s, h, _), dv_dim = q.shape, v.shape[-1]
+    o = torch.empty((b, s, h, dv_dim), dtype=torch.bfloat16, device=q.device)
+    lse = torch.empty((b, h, s), dtype=torch.float32, device=q.device)
+    attn_fwd_into(q, k, v, o, lse, softmax_scale, causal)
+    return o, lse
+
+
+def _mla_bwd_preprocess(out: torch.Tensor, dout: torch.Tensor):
+    """Phase 1: delta = rowsum(out * dout). Called once with combined_out."""
+    b, s, h, _ = out.shape
+    delta = torch.empty((b, h, s), dtype=torch.float32, device=out.device)
+    attn_bwd_delta_into(out, dout, delta)
+    return delta
+
+
+def _mla_bwd_dk_dv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
+                   lse: torch.Tensor, delta: torch.Tensor, softmax_scale: float, causal: bool = True):  # fmt: skip
+    """Phase 2: compute dK and dV using external lse and delta. Returns (dk, dv)."""
+    dk = torch.empty_like(k)
+    dv_out = torch.empty_like(v)
+    attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv_out, softmax_scale, causal)
+    return dk, dv_out
+
+
+def _mla_bwd_dq(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
+                lse: torch.Tensor, delta: torch.Tensor, softmax_scale: float, causal: bool = True):  # fmt: skip
+    """Phase 3: compute dQ using external lse and delta. Returns dq."""
+    dq_out = torch.empty_like(q)
+    attn_bwd_dq_into(q, k, v, dout, lse, delta, dq_out, softmax_scale, causal)
+    return dq_out
+
+
+class _CausalAttentionFunc(torch.autograd.Function):
+    """Single-device causal attention with the HIP kernels (what MLA.forward differentiates)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, softmax_scale):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        o, lse = _mla_fwd(q, k, v, softmax_scale, causal=True)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.softmax_scale = softmax_scale
+        return o
+
+    @staticmethod
+    def backward(ctx, grad_o):
+        q, k, v, o, lse = ctx.saved_tensors
+        grad_o = grad_o.contiguous()
+        delta = _mla_bwd_preprocess(o, grad_o)
+        dk, dv = _mla_bwd_dk_dv(q, k, v, grad_o, lse, delta, ctx.softmax_scale, causal=True)
+        dq = _mla_bwd_dq(q, k, v, grad_o, lse, delta, ctx.softmax_scale, causal=True)
+        return dq, dk, dv, None
+
+
+class MLA(nn.Module):
+    """
+    HIP implementation of the MLA operator (causal, BSHD layout); constructor and forward follow
+    pithtrain/operators/mla/pytorch.py:8-34 and pithtrain/operators/mla/triton.py:510-549.
+    """
+
+    def __init__(self, h: int, dq: int, dv: int, softmax_scale: float = 0.0):
+        super().__init__()
+        self.h = h
+        self.dq = dq
+        self.dv = dv
+        self.softmax_scale = softmax_scale if softmax_scale != 0.0 else math.sqrt(1.0 / dq)
+
+    @staticmethod
+    def autotune(b: int, s: int, h: int, dq: int, dv: int, softmax_scale: float,
+                 include_non_causal: bool = False) -> None:  # fmt: skip
+        """Kept for call-site compatibility (pithtrain/tasks/pretrain_language_model.py:497-501):
+        the HIP kernels are compiled ahead of time with fixed tilings, so there is nothing to tune;
+        only the head dims are validated, as the reference asserts them."""
+        assert (dq, dv) in SUPPORTED_HEAD_DIMS, (
+            f"HIP attention kernels support (dq, dv) in {SUPPORTED_HEAD_DIMS}, got dq={dq} and dv={dv}"
+        )
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        return _CausalAttentionFunc.apply(q, k, v, self.softmax_scale)
+
+
+__all__ = [
+    "MLA", "_mla_fwd", "_mla_bwd_preprocess", "_mla_bwd_dk_dv", "_mla_bwd_dq",
+    "attn_fwd_into", "attn_bwd_delta_into", "attn_bwd_dkdv_into", "attn_bwd_dq_into",
+]  # fmt: skip

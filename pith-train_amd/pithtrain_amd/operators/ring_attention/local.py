@@ -1,0 +1,288 @@
+"""
+One GPU's share of causal ring attention, computed without collectives.
+
+The reference ring (pithtrain/operators/ring_attention/standard.py:73-189, mla.py:47-149) runs
+cp_size steps on every rank; at each step the rank holds one K/V chunk, attends its local Q
+against it, merges the partial result into a running (out, lse) pair, and passes the chunk on.
+Here the chunks a rank would receive are handed in as a list (indexed by the rank that owns
+them), and the same per-step work runs back to back on one device: chunk attention forward,
+log2-domain combine, and in backward the per-chunk dQ/dK/dV against the combined LSE and
+delta = rowsum(dO*O) computed once.
+
+Two token layouts:
+
+  "contiguous"  the reference's: rank r owns tokens [r*S_l, (r+1)*S_l). It computes the causal
+                diagonal chunk and full attention against chunks 0..r-1 (standard.py:86-93), so
+                work grows with the rank (the imbalance noted at standard.py:16-18).
+  "zigzag"      the sequence is cut into 2C blocks and rank r owns blocks r and 2C-1-r, in that
+                order. Step 0 is plain causal attention over the local chunk. For a chunk of a
+                lower rank j < r only its first block is visible, to every local query; for a
+                chunk of a higher rank j > r the whole chunk is visible, but only to the second
+                local block. Every rank does the same amount of work.
+
+Running state follows the reference: partial results are merged in fp32 (the type promotion at
+mla.py:38) and rounded to bf16 once at the end (mla.py:78); here the last combine that touches a
+row range writes bf16 directly, which is the same single rounding. dQ is accumulated over steps
+in fp32 inside the dQ kernel's epilogue and rounded once (the reference adds bf16 partials,
+mla.py:116). dK/dV of every visited chunk are returned separately, zero where a chunk's rows were
+not visible; on a real ring those are what travels back to the owning ranks (standard.py:164-187).
+"""
+
+from dataclasses import dataclass
+from typing import List, Sequence, Tuple
+
+import torch
+
+from pithtrain_amd import _C
+from pithtrain_amd.operators.mla.hip import (
+    attn_bwd_delta_into,
+    attn_bwd_dkdv_into,
+    attn_bwd_dq_into,
+    attn_fwd_into,
+)
+from pithtrain_amd.operators.ring_attention.combine import cast_f32_bf16_into, combine_into
+
+LAYOUTS = ("contiguous", "zigzag")
+
+
+@dataclass(frozen=True)
+class RingStep:
+    """One step of a rank's ring: which chunk, which rows of each side take part, and the mask."""
+
+    kv_rank: int
+    causal: bool
+    q_rows: Tuple[int, int]  # [start, stop) within the local chunk
+    kv_rows: Tuple[int, int]  # [start, stop) within the visited chunk
+
+
+def ring_schedule(cp_rank: int, cp_size: int, s_local: int, layout: str = "contiguous") -> List[RingStep]:
+    """Steps rank `cp_rank` performs, in ring arrival order kv_rank = (cp_rank - step) % cp_size."""
+    assert layout in LAYOUTS, f"layout must be one of {LAYOUTS}, got {layout!r}"
+    assert 0 <= cp_rank < cp_size
+    full = (0, s_local)
+    steps = []
+    if layout == "zigzag":
+        assert s_local % 2 == 0, "zigzag needs an even local sequence length"
+        half = s_local // 2
+    for step in range(cp_size):
+        j = (cp_rank - step) % cp_size
+        if j == cp_rank:
+            steps.append(RingStep(j, True, full, full))
+        elif layout == "contiguous":
+            if j < cp_rank:
+                steps.append(RingStep(j, False, full, full))
+        elif j < cp_rank:
+            steps.append(RingStep(j, False, full, (0, half)))
+        else:
+            steps.append(RingStep(j, False, (half, s_local), full))
+    return steps
+
+
+def zigzag_split(x: torch.Tensor, cp_size: int, dim: int = 1) -> List[torch.Tensor]:
+    """Cuts a full-sequence tensor into the per-rank zigzag chunks [block r ; block 2C-1-r]."""
+    blocks = x.chunk(2 * cp_size, dim=dim)
+    assert len(blocks) == 2 * cp_size, "sequence length must be a multiple of 2 * cp_size"
+    return [torch.cat([blocks[r], blocks[2 * cp_size - 1 - r]], dim=dim).contiguous() for r in range(cp_size)]
+
+
+def zigzag_merge(chunks: Sequence[torch.Tensor], dim: int = 1) -> torch.Tensor:
+    """Inverse of zigzag_split."""
+    cp_size = len(chunks)
+    blocks = [None] * (2 * cp_size)
+    for r, c in enumerate(chunks):
+        first, second = c.chunk(2, dim=dim)
+        blocks[r], blocks[2 * cp_size - 1 - r] = first, second
+    return torch.cat(blocks, dim=dim)
+
+
+def _rows(t: torch.Tensor, rows: Tuple[int, int]) -> torch.Tensor:
+    """Row range of a [B, S, H, D] tensor (a view)."""
+    return t if rows == (0, t.shape[1]) else t[:, rows[0] : rows[1]]
+
+
+def _lse_rows(t: torch.Tensor, rows: Tuple[int, int]) -> torch.Tensor:
+    """Row range of a [B, H, S] tensor (a view)."""
+    return t if rows == (0, t.shape[2]) else t[:, :, rows[0] : rows[1]]
+
+
+class RingForward:
+    """Running (out, lse) of one rank's forward; feed it the schedule's steps in order."""
+
+    def __init__(self, q: torch.Tensor, dv_dim: int, softmax_scale: float, steps: Sequence[RingStep], layout: str):
+        assert q.is_contiguous(), "ring attention q is not contiguous"
+        B, S, H, _ = q.shape
+        self.q, self.scale, self.steps = q, softmax_scale, list(steps)
+        self.out = torch.empty((B, S, H, dv_dim), dtype=torch.bfloat16, device=q.device)
+        self.lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
+        # Row ranges are merged independently. `pending[r]` counts the merges still to come for
+        # range r; while it is non-zero the running value of the range lives in the fp32
+        # accumulator (or still in `out`, in bf16, before its first merge); the last merge of a
+        # range writes bf16 into `out`.
+        self.ranges = [(0, S)] if layout == "contiguous" else [(0, S // 2), (S // 2, S)]
+        self.pending = {r: sum(self._covers(st, r) for st in self.steps[1:]) for r in self.ranges}
+        self.in_acc = {r: False for r in self.ranges}
+        self.acc = None
+        if any(n > 1 for n in self.pending.values()):
+            self.acc = torch.empty((B, S, H, dv_dim), dtype=torch.float32, device=q.device)
+        self.step_out = self.step_lse = None
+        if len(self.steps) > 1:
+            self.step_out = torch.empty((B, S, H, dv_dim), dtype=torch.bfloat16, device=q.device)
+            self.step_lse = torch.empty(B * H * S, dtype=torch.float32, device=q.device)
+        self.done = 0
+
+    @staticmethod
+    def _covers(step: RingStep, r: Tuple[int, int]) -> bool:
+        return step.q_rows[0] <= r[0] and r[1] <= step.q_rows[1]
+
+    def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor) -> None:
+        assert st == self.steps[self.done], "ring steps must be fed in schedule order"
+        assert k_j.is_contiguous() and v_j.is_contiguous(), "ring attention k or v is not contiguous"
+        B, S, H, _ = self.q.shape
+        self.done += 1
+        if self.done == 1:
+            # Step 0 is the diagonal chunk and covers every local row: merging it into the
+            # reference's initial state (zeros, finfo.min) returns it unchanged, so it is written
+            # straight into the running tensors.
+            assert st.causal and st.q_rows == (0, S)
+            attn_fwd_into(self.q, k_j, v_j, self.out, self.lse, self.scale, True)
+            return
+        n_q = st.q_rows[1] - st.q_rows[0]
+        so = self.step_out[:, :n_q]
+        sl = self.step_lse[: B * H * n_q].view(B, H, n_q)
+        attn_fwd_into(_rows(self.q, st.q_rows), _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows), so, sl,
+                      self.scale, False)  # fmt: skip
+        # Ranges in the same state are merged by one launch.
+        groups = {}
+        for r in self.ranges:
+            if self._covers(st, r):
+                groups.setdefault((self.in_acc[r], self.pending[r] == 1), []).append(r)
+        for (from_acc, last), rs in groups.items():
+            lo, hi = rs[0][0], rs[-1][1]
+            rel = (lo - st.q_rows[0], hi - st.q_rows[0])
+            src = _rows(self.acc if from_acc else self.out, (lo, hi))
+            dst = _rows(self.out if last else self.acc, (lo, hi))
+            run_lse = _lse_rows(self.lse, (lo, hi))
+            combine_into(src, run_lse, _rows(so, rel), _lse_rows(sl, rel), dst, run_lse, _C.PITH_BASE_2)
+            for r in rs:
+                self.pending[r] -= 1
+                self.in_acc[r] = not last
+
+    def result(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        assert self.done == len(self.steps), "not every ring step has run"
+        return self.out, self.lse
+
+
+class RingBackward:
+    """Gradient state of one rank's backward; feed it the schedule's steps in order."""
+
+    def __init__(self, dout, q, out, lse, softmax_scale: float, steps: Sequence[RingStep]):
+        self.dout = dout.contiguous()
+        self.q, self.lse, self.scale, self.steps = q, lse, softmax_scale, list(steps)
+        B, S, H, _ = q.shape
+        # delta from the COMBINED output, once (pithtrain/operators/ring_attention/mla.py:101).
+        self.delta = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
+        attn_bwd_delta_into(out, self.dout, self.delta)
+        self.dq = torch.empty_like(q)
+        single = len(self.steps) == 1
+        self.dq_acc = self.dq if single else torch.empty(q.shape, dtype=torch.float32, device=q.device)
+        self.done = 0
+
+    def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor):
+        """Returns (dk_j, dv_j), this rank's contribution to chunk st.kv_rank's gradients."""
+        assert st == self.steps[self.done], "ring steps must be fed in schedule order"
+        dk_j, dv_j = torch.empty_like(k_j), torch.empty_like(v_j)
+        if st.kv_rows != (0, k_j.shape[1]):  # rows of the chunk this rank cannot see get no gradient
+            for t in (dk_j, dv_j):
+                t[:, : st.kv_rows[0]].zero_()
+                t[:, st.kv_rows[1] :].zero_()
+        qs, ds = _rows(self.q, st.q_rows), _rows(self.dout, st.q_rows)
+        ks, vs = _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows)
+        ls, dl = _lse_rows(self.lse, st.q_rows), _lse_rows(self.delta, st.q_rows)
+        attn_bwd_dkdv_into(qs, ks, vs, ds, ls, dl, _rows(dk_j, st.kv_rows), _rows(dv_j, st.kv_rows),
+                           self.scale, st.causal)  # fmt: skip
+        # Step 0 covers every row and initialises the accumulator; later steps add to their rows.
+        attn_bwd_dq_into(qs, ks, vs, ds, ls, dl, _rows(self.dq_acc, st.q_rows), self.scale, st.causal,
+                         accumulate=self.done > 0)  # fmt: skip
+        self.done += 1
+        return dk_j, dv_j
+
+    def finish(self) -> torch.Tensor:
+        assert self.done == len(self.steps), "not every ring step has run"
+        if self.dq_acc is not self.dq:
+            cast_f32_bf16_into(self.dq_acc, self.dq)
+        return self.dq
+
+
+def ring_forward_local(
+    q: torch.Tensor, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor],
+    softmax_scale: float, cp_rank: int, cp_size: int, layout: str = "contiguous",
+) -> Tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
+    """Forward of rank `cp_rank`: returns (out bf16 [B, S_l, Hq, Dv], lse fp32 base-2 [B, Hq, S_l]).
+
+    k_chunks[j] / v_chunks[j] are the K/V chunks owned by rank j (entries the schedule never
+    visits may be None)."""
+    steps = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
+    fwd = RingForward(q, v_chunks[cp_rank].shape[-1], softmax_scale, steps, layout)
+    for st in steps:
+        fwd.run_step(st, k_chunks[st.kv_rank], v_chunks[st.kv_rank])
+    return fwd.result()
+
+
+def ring_backward_local(
+    dout: torch.Tensor, q: torch.Tensor, out: torch.Tensor, lse: torch.Tensor,
+    k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor],
+    softmax_scale: float, cp_rank: int, cp_size: int, layout: str = "contiguous",
+):  # fmt: skip
+    """Backward of rank `cp_rank`. Returns (dq, dk_list, dv_list): dq bf16 like q; dk_list[j] and
+    dv_list[j] are this rank's contribution to the gradients of chunk j (None if never visited)."""
+    steps = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
+    bwd = RingBackward(dout, q, out, lse, softmax_scale, steps)
+    dk_list: List[torch.Tensor] = [None] * cp_size
+    dv_list: List[torch.Tensor] = [None] * cp_size
+    for st in steps:
+        dk_list[st.kv_rank], dv_list[st.kv_rank] = bwd.run_step(st, k_chunks[st.kv_rank], v_chunks[st.kv_rank])
+    return bwd.finish(), dk_list, dv_list
+
+
+class RingAttentionLocalFunc(torch.autograd.Function):
+    """autograd wrapper of one rank's ring share; gradients flow to q and to every visited chunk."""
+
+    @staticmethod
+    def forward(ctx, q, softmax_scale, cp_rank, cp_size, layout, *kv):
+        assert len(kv) == 2 * cp_size, "expected cp_size K chunks followed by cp_size V chunks"
+        k_chunks, v_chunks = list(kv[:cp_size]), list(kv[cp_size:])
+        out, lse = ring_forward_local(q, k_chunks, v_chunks, softmax_scale, cp_rank, cp_size, layout)
+        visited = sorted({st.kv_rank for st in ring_schedule(cp_rank, cp_size, q.shape[1], layout)})
+        ctx.save_for_backward(q, out, lse, *[k_chunks[j] for j in visited], *[v_chunks[j] for j in visited])
+        ctx.visited = visited
+        ctx.conf = (softmax_scale, cp_rank, cp_size, layout)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        softmax_scale, cp_rank, cp_size, layout = ctx.conf
+        saved = ctx.saved_tensors
+        q, out, lse = saved[0], saved[1], saved[2]
+        n = len(ctx.visited)
+        k_chunks, v_chunks = [None] * cp_size, [None] * cp_size
+        for i, j in enumerate(ctx.visited):
+            k_chunks[j], v_chunks[j] = saved[3 + i], saved[3 + n + i]
+        dq, dk_list, dv_list = ring_backward_local(
+            dout, q, out, lse, k_chunks, v_chunks, softmax_scale, cp_rank, cp_size, layout
+        )
+        return (dq, None, None, None, None, *dk_list, *dv_list)
+
+
+def ring_attention_local(
+    q: torch.Tensor, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor],
+    softmax_scale: float, cp_rank: int, cp_size: int, layout: str = "contiguous",
+) -> torch.Tensor:  # fmt: skip
+    """Differentiable one-GPU ring share for either model family (head dims pick the kernels)."""
+    assert len(k_chunks) == cp_size and len(v_chunks) == cp_size
+    # Chunks the schedule never visits may be None; autograd needs tensors, so they are replaced
+    # by empty placeholders that receive no gradient.
+    visited = {st.kv_rank for st in ring_schedule(cp_rank, cp_size, q.shape[1], layout)}
+    empty = q.new_empty(0)
+    ks = [k_chunks[j] if j in visited else empty for j in range(cp_size)]
+    vs = [v_chunks[j] if j in visited else empty for j in range(cp_size)]
+    return RingAttentionLocalFunc.apply(q, softmax_scale, cp_rank, cp_size, layout, *ks, *vs)

@@ -51,6 +51,16 @@ struct Vec8<float> {
   }
 };
 
+// (w1*x + w2*y) * rinv with each product rounded on its own (no fused multiply-add), as the
+// reference's eager expression evaluates it: the result is then bit-identical when the two
+// partials are swapped.
+__device__ __forceinline__ float merge_element(float w1, float x, float w2, float y, float rinv) {
+#pragma clang fp contract(off)
+  const float a = w1 * x;
+  const float b = w2 * y;
+  return (a + b) * rinv;
+}
+
 struct CombineParams {
   const void* out1;
   const float* lse1;
@@ -73,7 +83,7 @@ struct CombineParams {
 //          with 16-byte accesses; thread t owns chunks t, t+256, ...
 template <typename T1, typename T2, typename TO>
 __global__ __launch_bounds__(kCombineThreads) void combine_kernel(CombineParams p) {
-  extern __shared__ float weights[];  // [rows][2], rows = tile_s * H, row = s_local * H + h
+  extern __shared__ float weights[];  // [rows][3] = (w1, w2, 1/(w1+w2)), rows = tile_s * H, row = s_local * H + h
   const int b = blockIdx.y;
   const int64_t s0 = (int64_t)blockIdx.x * p.tile_s;
   const int ts = (int)min((int64_t)p.tile_s, p.S - s0);
@@ -87,29 +97,30 @@ __global__ __launch_bounds__(kCombineThreads) void combine_kernel(CombineParams 
     const float a = l1[h * p.lse1_hs + sl];
     const float c = l2[h * p.lse2_hs + sl];
     const float m = fmaxf(a, c);
-    float w1, w2, lse;
+    float w1, w2, rinv, lse;
     if (m == -INFINITY) {
       // Both partials are empty: the reference yields NaN here (-inf - -inf); an empty
       // result (weights 0, lse -inf) is returned instead. The ring never produces this case.
       w1 = 0.f;
       w2 = 0.f;
+      rinv = 0.f;
       lse = -INFINITY;
     } else {
-      float e1, e2;
       if (p.base_e) {
-        e1 = expf(a - m);
-        e2 = expf(c - m);
+        w1 = expf(a - m);
+        w2 = expf(c - m);
       } else {
-        e1 = exp2f(a - m);
-        e2 = exp2f(c - m);
+        w1 = exp2f(a - m);
+        w2 = exp2f(c - m);
       }
-      const float sum = e1 + e2;
-      w1 = e1 / sum;
-      w2 = e2 / sum;
+      const float sum = w1 + w2;
+      rinv = 1.f / sum;
       lse = m + (p.base_e ? logf(sum) : log2f(sum));
     }
-    weights[2 * (sl * p.H + h)] = w1;
-    weights[2 * (sl * p.H + h) + 1] = w2;
+    float* w = weights + 3 * (sl * p.H + h);
+    w[0] = w1;
+    w[1] = w2;
+    w[2] = rinv;
     lo[h * p.lse_out_hs + sl] = lse;
   }
   __syncthreads();
@@ -137,14 +148,12 @@ __global__ __launch_bounds__(kCombineThreads) void combine_kernel(CombineParams 
       const int c = c0 + u * kCombineThreads;
       if (c < chunks) {
         const int row = c / p.D8;
-        const float w1 = weights[2 * row], w2 = weights[2 * row + 1];
+        const float w1 = weights[3 * row], w2 = weights[3 * row + 1], rinv = weights[3 * row + 2];
         Vec8<TO> r;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float v0 = w1 * x[u].get(2 * j) + w2 * y[u].get(2 * j);
-          const float v1 = w1 * x[u].get(2 * j + 1) + w2 * y[u].get(2 * j + 1);
-          r.set_pair(j, v0, v1);
-        }
+        for (int j = 0; j < 4; ++j)
+          r.set_pair(j, merge_element(w1, x[u].get(2 * j), w2, y[u].get(2 * j), rinv),
+                     merge_element(w1, x[u].get(2 * j + 1), w2, y[u].get(2 * j + 1), rinv));
         r.store(oo + (int64_t)c * 8);
       }
     }
@@ -263,7 +272,7 @@ extern "C" int pith_combine(const pith_combine_args* a, pith_stream_t stream) {
   p.lse_out_bs = a->lse_out_bs; p.lse_out_hs = a->lse_out_hs;
   p.tile_s = pick_tile_s(a->B, a->S, a->H, 4096);
   const dim3 grid((unsigned)((a->S + p.tile_s - 1) / p.tile_s), (unsigned)a->B);
-  const size_t lds = (size_t)p.tile_s * p.H * 2 * sizeof(float);
+  const size_t lds = (size_t)p.tile_s * p.H * 3 * sizeof(float);
   hipStream_t st = (hipStream_t)stream;
   if (a->dtype1 == PITH_BF16) {
     if (a->dtype2 == PITH_BF16) launch_combine_t2<__bf16, __bf16>(p, a->dtype_out, grid, lds, st);

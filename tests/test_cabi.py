@@ -1,0 +1,145 @@
+"""The C-ABI library on a machine without a GPU: it loads, exports every symbol include/pith_hip.h
+declares, its argument structs have the layout the Python binding assumes, and every entry point
+rejects bad arguments with an error code before touching the device."""
+
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pith_hip.h")
+
+from pithtrain_amd import _C  # noqa: E402
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pith_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _C.lib()
+    declared = _declared_symbols()
+    assert len(declared) >= 9
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in pith_hip.h but not exported"
+    assert sorted(_C.SYMBOLS) == declared, "python binding table and header disagree"
+    assert lib.pith_version() >= 100
+    assert lib.pith_error_name(-2) == b"PITH_ERR_BAD_SHAPE"
+
+
+def test_struct_layouts_match_the_header(tmp_path):
+    """sizeof/offsetof from a C compile of the header against the ctypes Structures."""
+    pairs = {
+        "pith_combine_args": _C.CombineArgs,
+        "pith_attn_fwd_args": _C.AttnFwdArgs,
+        "pith_attn_delta_args": _C.AttnDeltaArgs,
+        "pith_attn_bwd_args": _C.AttnBwdArgs,
+    }
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "pith_hip.h"', "int main(void){"]
+    for cname, st in pairs.items():
+        lines.append(f'printf("{cname} %zu\\n", sizeof({cname}));')
+        for fname, _ in st._fields_:
+            lines.append(f'printf("{cname}.{fname} %zu\\n", offsetof({cname}, {fname}));')
+    lines.append("return 0;}")
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    got = dict(line.split() for line in out.strip().splitlines())
+    for cname, st in pairs.items():
+        assert int(got[cname]) == ctypes.sizeof(st), cname
+        for fname, _ in st._fields_:
+            assert int(got[f"{cname}.{fname}"]) == getattr(st, fname).offset, f"{cname}.{fname}"
+
+
+def _fwd_args(**kw):
+    base = dict(q=16, k=16, v=16, o=16, lse=16, B=1, Sq=64, Skv=64, Hq=4, Hkv=2, Dqk=128, Dv=128,
+                q_bs=64 * 4 * 128, k_bs=64 * 2 * 128, v_bs=64 * 2 * 128, o_bs=64 * 4 * 128,
+                lse_bs=4 * 64, lse_hs=64, scale=0.088, causal=0)  # fmt: skip
+    base.update(kw)
+    return _C.AttnFwdArgs(**base)
+
+
+@pytest.mark.parametrize(
+    "kw,code",
+    [
+        (dict(q=None), _C.PITH_ERR_NULL_POINTER),
+        (dict(Sq=0), _C.PITH_ERR_BAD_SHAPE),
+        (dict(Hq=3), _C.PITH_ERR_BAD_SHAPE),
+        (dict(causal=1, Skv=32), _C.PITH_ERR_UNSUPPORTED),
+        (dict(Dqk=96), _C.PITH_ERR_UNSUPPORTED),
+        (dict(Dqk=192, Dv=192), _C.PITH_ERR_UNSUPPORTED),
+        (dict(k=8), _C.PITH_ERR_MISALIGNED),
+        (dict(q_bs=100), _C.PITH_ERR_MISALIGNED),
+    ],
+)
+def test_attn_fwd_rejects_bad_arguments(kw, code):
+    lib = _C.lib()
+    rc = lib.pith_attn_fwd(ctypes.byref(_fwd_args(**kw)), None)
+    assert rc == code, lib.pith_last_error()
+    assert lib.pith_last_error().startswith(b"pith_attn_fwd")
+    with pytest.raises(_C.PithError) as e:
+        _C.check(rc)
+    assert e.value.code == code
+
+
+def test_null_args_struct_is_rejected_everywhere():
+    lib = _C.lib()
+    for name in ("pith_combine", "pith_attn_fwd", "pith_attn_bwd_delta", "pith_attn_bwd_dkdv", "pith_attn_bwd_dq"):
+        assert getattr(lib, name)(None, None) == _C.PITH_ERR_NULL_POINTER, name
+    assert lib.pith_cast_f32_bf16(None, None, 8, None) == _C.PITH_ERR_NULL_POINTER
+    assert lib.pith_cast_f32_bf16(16, 16, 12, None) == _C.PITH_ERR_BAD_SHAPE
+
+
+def test_combine_and_bwd_validation():
+    lib = _C.lib()
+    c = _C.CombineArgs(out1=16, lse1=16, out2=16, lse2=16, out=16, lse_out=16, dtype1=0, dtype2=1, dtype_out=1,
+                       base=0, B=1, S=8, H=2, D=128, out1_bs=2048, out2_bs=2048, out_bs=2048, lse1_bs=16, lse1_hs=8,
+                       lse2_bs=16, lse2_hs=8, lse_out_bs=16, lse_out_hs=8)  # fmt: skip
+    c.dtype2 = 7
+    assert lib.pith_combine(ctypes.byref(c), None) == _C.PITH_ERR_BAD_DTYPE
+    c.dtype2, c.base = 1, 5
+    assert lib.pith_combine(ctypes.byref(c), None) == _C.PITH_ERR_BAD_DTYPE
+    c.base, c.D = 0, 100
+    assert lib.pith_combine(ctypes.byref(c), None) == _C.PITH_ERR_BAD_SHAPE
+    b = _C.AttnBwdArgs(q=16, k=16, v=16, dout=16, lse=16, delta=16, dq=None, dk=16, dv=16, B=1, Sq=64, Skv=64, Hq=4,
+                       Hkv=4, Dqk=128, Dv=128, scale=0.1)  # fmt: skip
+    assert lib.pith_attn_bwd_dq(ctypes.byref(b), None) == _C.PITH_ERR_NULL_POINTER  # dq missing
+    b.dk = None
+    assert lib.pith_attn_bwd_dkdv(ctypes.byref(b), None) == _C.PITH_ERR_NULL_POINTER
+    d = _C.AttnDeltaArgs(o=16, dout=16, delta=16, B=1, S=8, H=2, D=96)
+    assert lib.pith_attn_bwd_delta(ctypes.byref(d), None) == _C.PITH_ERR_UNSUPPORTED
+
+
+def test_operators_refuse_cpu_tensors():
+    """No CPU fallback: the product path raises instead of computing somewhere else."""
+    import torch
+
+    from pithtrain_amd.operators.mla.hip import _mla_fwd
+    from pithtrain_amd.operators.ring_attention.mla import _online_softmax_combine_log2
+
+    q = torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="need tensors on a GPU"):
+        _mla_fwd(q, q, q, 0.1, causal=True)
+    lse = torch.zeros(1, 2, 64)
+    with pytest.raises(RuntimeError, match="need tensors on a GPU"):
+        _online_softmax_combine_log2(q, lse, q, lse)
+
+
+def test_ring_schedule_matches_oracle_schedule():
+    """Host logic: the product's step schedule equals the oracle's independent restatement."""
+    from oracle import ring_oracle as R
+    from pithtrain_amd.operators.ring_attention.local import ring_schedule
+
+    for layout in ("contiguous", "zigzag"):
+        for C in (1, 2, 3, 4, 8):
+            for r in range(C):
+                ours = [(s.kv_rank, s.causal, s.q_rows, s.kv_rows) for s in ring_schedule(r, C, 64, layout)]
+                assert ours == R._steps(r, C, 64, layout)

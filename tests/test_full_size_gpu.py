@@ -1,0 +1,99 @@
+"""Parity at BASELINE sizes. The dense oracle cannot cover 32K-131K tokens in seconds, so each
+case runs the whole ring share on the GPU and checks SAMPLED rows against exact full-sequence
+causal attention evaluated only for those rows (cost: rows x total keys):
+
+  O, LSE2, dQ  : sampled local query rows against every key of the global sequence they may see;
+  dK_j, dV_j   : sampled key rows of every visited chunk against every local query row, using the
+                 kernel's LSE2 and delta (themselves checked on the sampled query rows).
+
+Inputs follow BASELINE's recipe: CPU generator seed 42, q/k/v ~ N(0,1)/sqrt(Dqk), dO ~ N(0,1)."""
+
+import pytest
+import torch
+
+from helpers import check_bf16_result, check_lse
+from oracle import ring_oracle as R
+from pithtrain_amd.operators.ring_attention.local import ring_backward_local, ring_forward_local
+
+pytestmark = pytest.mark.gpu
+
+CASES = [  # Hq, Hkv, Dqk, Dv, S_local, C, rank
+    pytest.param(32, 4, 128, 128, 8192, 4, 1, id="qwen3-32k-c4-r1"),
+    pytest.param(16, 16, 192, 128, 4096, 4, 1, id="mla-16k-c4-r1"),
+    pytest.param(64, 4, 128, 128, 16384, 8, 3, id="long-131k-c8-r3"),
+]
+
+
+def make_inputs(Hq, Hkv, Dqk, Dv, S_l, C, seed=42):
+    g = torch.Generator().manual_seed(seed)
+    s = Dqk**-0.5
+    q = (torch.randn(1, S_l, Hq, Dqk, generator=g) * s).to(torch.bfloat16)
+    ks = [(torch.randn(1, S_l, Hkv, Dqk, generator=g) * s).to(torch.bfloat16) for _ in range(C)]
+    vs = [(torch.randn(1, S_l, Hkv, Dv, generator=g) * s).to(torch.bfloat16) for _ in range(C)]
+    dout = torch.randn(1, S_l, Hq, Dv, generator=g).to(torch.bfloat16)
+    return q, ks, vs, dout
+
+
+@pytest.mark.parametrize("Hq,Hkv,Dqk,Dv,S_l,C,r", CASES)
+def test_zigzag_share_sampled_rows(gpu, Hq, Hkv, Dqk, Dv, S_l, C, r):
+    layout = "zigzag"
+    scale = Dqk**-0.5
+    q, ks, vs, dout = make_inputs(Hq, Hkv, Dqk, Dv, S_l, C)
+    qd, dod = q.to(gpu), dout.to(gpu)
+    kd, vd = [c.to(gpu) for c in ks], [c.to(gpu) for c in vs]
+    out, lse = ring_forward_local(qd, kd, vd, scale, r, C, layout)
+    dq, dks, dvs = ring_backward_local(dod, qd, out, lse, kd, vd, scale, r, C, layout)
+    torch.cuda.synchronize()
+    assert all(torch.isfinite(t.float()).all() for t in (out, lse, dq))
+
+    # ---- sampled query rows: first/last rows of both local blocks plus random ones
+    g = torch.Generator().manual_seed(1)
+    half = S_l // 2
+    rows = torch.unique(torch.cat([torch.tensor([0, 1, half - 1, half, half + 1, S_l - 1]),
+                                   torch.randint(0, S_l, (18 if C * S_l > 65536 else 42,), generator=g)]))  # fmt: skip
+    pos_local = R.token_positions(r, C, S_l, layout)
+    key_pos = torch.cat([R.token_positions(j, C, S_l, layout) for j in range(C)])  # position of every key, chunk-major
+    k_all, v_all = torch.cat(ks, 1).double(), torch.cat(vs, 1).double()  # [1, C*S_l, Hkv, D]
+    grp = Hq // Hkv
+    n = len(rows)
+    qs = q[:, rows].double().reshape(1, n, Hkv, grp, Dqk)
+    dos = dout[:, rows].double().reshape(1, n, Hkv, grp, Dv)
+    s = torch.einsum("bihgd,bjhd->bhgij", qs, k_all) * (scale * R.LOG2E)
+    visible = key_pos.unsqueeze(0) <= pos_local[rows].unsqueeze(1)  # [rows, keys]
+    s = s.masked_fill(~visible, float("-inf"))
+    ln2 = torch.log(torch.tensor(2.0, dtype=torch.float64))
+    lse_ref = torch.logsumexp(s * ln2, -1) / ln2  # [1, Hkv, grp, n]
+    p = torch.exp2(s - lse_ref.unsqueeze(-1))
+    del s
+    o_ref = torch.einsum("bhgij,bjhd->bihgd", p, v_all)
+    check_lse(lse[:, :, rows], lse_ref.reshape(1, Hq, n), "LSE2 (sampled rows)")
+    check_bf16_result(out[:, rows], o_ref.reshape(1, n, Hq, Dv), "O (sampled rows)")
+    delta_ref = (o_ref * dos).sum(-1).permute(0, 2, 3, 1)  # [1, Hkv, grp, n]
+    dp = torch.einsum("bihgd,bjhd->bhgij", dos, v_all)
+    ds = p * (dp - delta_ref.unsqueeze(-1)) * scale
+    del p, dp
+    dq_ref = torch.einsum("bhgij,bjhd->bihgd", ds, k_all).reshape(1, n, Hq, Dqk)
+    del ds
+    check_bf16_result(dq[:, rows], dq_ref, "dQ (sampled rows)", otol=1e-3)
+
+    # ---- sampled key rows of every chunk: contribution of all local queries
+    delta_gpu = (out.float() * dod.float()).sum(-1).transpose(1, 2)  # [1, Hq, S_l]
+    lse_gpu = lse
+    for j in range(C):
+        krows = torch.unique(torch.cat([torch.tensor([0, half - 1, half, S_l - 1]),
+                                        torch.randint(0, S_l, (12,), generator=g)]))  # fmt: skip
+        kj = kd[j][:, krows].float().repeat_interleave(grp, 2)
+        vj = vd[j][:, krows].float().repeat_interleave(grp, 2)
+        sj = torch.einsum("bihd,bjhd->bhij", qd.float(), kj) * (scale * R.LOG2E)  # [1, Hq, S_l, n]
+        vis = (R.token_positions(j, C, S_l, layout)[krows].unsqueeze(0) <= pos_local.unsqueeze(1)).to(gpu)
+        pj = torch.exp2(sj - lse_gpu.unsqueeze(-1)) * vis
+        dv_ref = torch.einsum("bhij,bihd->bjhd", pj, dod.float())
+        dpj = torch.einsum("bihd,bjhd->bhij", dod.float(), vj)
+        dsj = pj * (dpj - delta_gpu.unsqueeze(-1)) * scale
+        dk_ref = torch.einsum("bhij,bihd->bjhd", dsj, qd.float())
+        dk_ref = dk_ref.reshape(1, len(krows), Hkv, grp, Dqk).sum(3)
+        dv_ref = dv_ref.reshape(1, len(krows), Hkv, grp, Dv).sum(3)
+        check_bf16_result(dks[j][:, krows], dk_ref, f"dK chunk {j} (sampled rows)", otol=2e-3)
+        check_bf16_result(dvs[j][:, krows], dv_ref, f"dV chunk {j} (sampled rows)", otol=2e-3)
+        if j < r:  # only the first block of a lower rank's chunk is visible
+            assert not dks[j][:, half:].any() and not dvs[j][:, half:].any()

@@ -1,0 +1,261 @@
+#!/usr/bin/env python3
+"""Benchmark of the ring-attention hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step is one forward + backward pass of one GPU's share of causal ring attention at the
+Qwen3-30B-A3B shape (32 q heads / 4 kv heads, head dim 128, 32768 tokens as 4 zigzag chunks of 8192,
+rank 1 of 4): 4 chunk-attention forwards, 3 log2 combines, delta, 4 dK/dV and 4 dQ launches.
+Inputs are synthetic (CPU generator, seed 42; q/k/v ~ N(0,1)/sqrt(128), dO ~ N(0,1)) and resident in
+HBM before the timed region. One JSON line is printed:
+
+  value      algorithmic TFLOP/s of the whole step: 2*(Dqk+Dv)*E*Hq forward + 2*(3Dqk+2Dv)*E*Hq backward
+             with E = C*S_l^2/2 score entries per head (5 backward matmuls; recomputation not counted)
+  roofline   the dominant kernel (non-causal dK/dV), timed per launch with events on the launch stream
+  combine    the log2 combine at [1,4096,32,128] bf16+bf16 -> fp32 over rotating buffers, GB/s of
+             algorithmic bytes against the 8 TB/s HBM peak, with its own roofline
+  cpu_baseline  the oracle's eager-PyTorch restatement of the same ring share, timed on the host
+             cores over one kv-head group (8 of the 32 query heads)
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "pith-train_amd"))
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+HBM_PEAK_GBPS = 8000.0
+
+HQ, HKV, DQK, DV, S_LOCAL, CP, RANK = 32, 4, 128, 128, 8192, 4, 1
+LAYOUT = "zigzag"
+
+
+def make_inputs(torch, device):
+    g = torch.Generator().manual_seed(42)
+    s = DQK**-0.5
+    q = (torch.randn(1, S_LOCAL, HQ, DQK, generator=g) * s).to(torch.bfloat16)
+    ks = [(torch.randn(1, S_LOCAL, HKV, DQK, generator=g) * s).to(torch.bfloat16) for _ in range(CP)]
+    vs = [(torch.randn(1, S_LOCAL, HKV, DV, generator=g) * s).to(torch.bfloat16) for _ in range(CP)]
+    dout = torch.randn(1, S_LOCAL, HQ, DV, generator=g).to(torch.bfloat16)
+    host = (q, ks, vs, dout)
+    dev = (q.to(device), [c.to(device) for c in ks], [c.to(device) for c in vs], dout.to(device))
+    return host, dev
+
+
+def flops_per_step():
+    entries = CP * S_LOCAL * S_LOCAL // 2  # per head, this rank's zigzag share
+    fwd = 2 * (DQK + DV) * entries * HQ
+    bwd = 2 * (3 * DQK + 2 * DV) * entries * HQ
+    return fwd, bwd
+
+
+def time_events(torch, fn, reps):
+    """Average milliseconds of fn() over `reps` calls, bracketed by events on the current stream."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def bench_ring(torch, args, dev_inputs):
+    from pithtrain_amd.operators.mla.hip import attn_bwd_dkdv_into
+    from pithtrain_amd.operators.ring_attention.local import (
+        ring_backward_local,
+        ring_forward_local,
+        ring_schedule,
+    )
+
+    q, ks, vs, dout = dev_inputs
+    scale = DQK**-0.5
+
+    def forward():
+        return ring_forward_local(q, ks, vs, scale, RANK, CP, LAYOUT)
+
+    def step():
+        out, lse = forward()
+        return ring_backward_local(dout, q, out, lse, ks, vs, scale, RANK, CP, LAYOUT)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    ms_fwd = time_events(torch, forward, args.steps)
+    out, lse = forward()
+    ms_bwd = time_events(torch, lambda: ring_backward_local(dout, q, out, lse, ks, vs, scale, RANK, CP, LAYOUT), args.steps)
+
+    # Dominant kernel: the non-causal dK/dV launch (3 per step; every one covers S_l^2/2 score
+    # entries per query head and performs 4 of the 5 algorithmic backward products).
+    from pithtrain_amd.operators.mla.hip import attn_bwd_delta_into
+
+    delta = torch.empty_like(lse)
+    attn_bwd_delta_into(out, dout, delta)
+    st = [s for s in ring_schedule(RANK, CP, S_LOCAL, LAYOUT) if not s.causal]
+    launches = []
+    for s in st:
+        k_j, v_j = ks[s.kv_rank][:, s.kv_rows[0] : s.kv_rows[1]], vs[s.kv_rank][:, s.kv_rows[0] : s.kv_rows[1]]
+        rows = slice(s.q_rows[0], s.q_rows[1])
+        dk, dv = torch.empty_like(k_j), torch.empty_like(v_j)
+        launches.append((q[:, rows], k_j, v_j, dout[:, rows], lse[:, :, rows], delta[:, :, rows], dk, dv))
+
+    def dkdv_launches():
+        for a in launches:
+            attn_bwd_dkdv_into(*a, scale, False)
+
+    dkdv_launches()
+    ms_dkdv = time_events(torch, dkdv_launches, args.steps) / len(launches)
+    entries = (S_LOCAL * S_LOCAL // 2) * HQ
+    dkdv_flops = 2 * (2 * DQK + 2 * DV) * entries
+    return ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops
+
+
+def bench_combine(torch, device, reps=50):
+    from pithtrain_amd.operators.ring_attention.combine import combine_into
+
+    B, S, H, D = 1, 4096, 32, 128
+    g = torch.Generator().manual_seed(42)
+    sets = []
+    for _ in range(4):  # 4 x 129.5 MiB > the 256 MiB last-level cache
+        o1 = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(device)
+        o2 = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(device)
+        l1 = (torch.rand(B, H, S, generator=g) * 16 - 4).to(device)
+        l2 = (torch.rand(B, H, S, generator=g) * 16 - 4).to(device)
+        out = torch.empty(B, S, H, D, dtype=torch.float32, device=device)
+        lse = torch.empty(B, H, S, dtype=torch.float32, device=device)
+        sets.append((o1, l1, o2, l2, out, lse))
+    nbytes = sum(t.numel() * t.element_size() for t in sets[0])
+    it = [0]
+
+    def one():
+        combine_into(*sets[it[0] % len(sets)])
+        it[0] += 1
+
+    for _ in range(8):
+        one()
+    ms = time_events(torch, one, reps)
+    host = [t.cpu() for t in sets[0][:4]]
+    return ms, nbytes, host
+
+
+def cpu_baseline_ring(torch, host_inputs):
+    from oracle import ring_oracle as R
+
+    q, ks, vs, dout = host_inputs
+    heads = (0, HQ // HKV)  # one kv-head group
+    t0 = time.perf_counter()
+    R.cpu_ring_fwd_bwd(q, ks, vs, dout, DQK**-0.5, RANK, CP, LAYOUT, heads=heads, q_block=1024)
+    dt = time.perf_counter() - t0
+    fwd, bwd = flops_per_step()
+    sample_flops = (fwd + bwd) * (heads[1] - heads[0]) / HQ
+    return sample_flops / dt / 1e12, dt
+
+
+def cpu_baseline_combine(torch, host, nbytes, reps=5):
+    from oracle import ring_oracle as R
+
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        R.combine_log2(*host)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return nbytes / times[len(times) // 2] / 1e9
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit(
+            "bench.py measures one GPU's share of the ring (no collectives are part of this build); "
+            f"--gpus {args.gpus} is not supported, run with --gpus 1"
+        )
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X: no GPU is visible")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    host_inputs, dev_inputs = make_inputs(torch, device)
+    ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops = bench_ring(torch, args, dev_inputs)
+    fwd_flops, bwd_flops = flops_per_step()
+    tflops = (fwd_flops + bwd_flops) / (ms_step * 1e-3) / 1e12
+    ms_comb, comb_bytes, comb_host = bench_combine(torch, device)
+    comb_gbps = comb_bytes / (ms_comb * 1e-3) / 1e9
+
+    cores = torch.get_num_threads()
+    cpu = None
+    combine_cpu = None
+    if not args.no_cpu_baseline:
+        cpu_tflops, cpu_s = cpu_baseline_ring(torch, host_inputs)
+        cpu = {
+            "value": round(cpu_tflops, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"same workload restricted to one kv-head group (8 of {HQ} query heads), all rows, fp32 eager "
+                      f"PyTorch, {cpu_s:.1f} s; os.cpu_count()={os.cpu_count()}",
+        }  # fmt: skip
+        combine_cpu = {
+            "value": round(cpu_baseline_combine(torch, comb_host, comb_bytes), 2), "unit": "GB/s", "cores": cores,
+            "kind": "port", "sample": "full [1,4096,32,128] combine, eager PyTorch, median of 5",
+        }  # fmt: skip
+
+    dkdv_tflops = dkdv_flops / (ms_dkdv * 1e-3) / 1e12
+    line = {
+        "metric": "ring-attn fwd+bwd causal TFLOP/s (Qwen3-30B-A3B, 32K)",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "GQA ring share fwd+bwd: 32 q / 4 kv heads, head dim 128, S=32768 as 4 zigzag chunks of "
+                        "8192 looped locally (rank 1), B=1, incl. log2 combines and delta",
+            "layout": LAYOUT, "cp_size": CP, "cp_rank": RANK, "s_local": S_LOCAL,
+        },  # fmt: skip
+        "frac_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+        "fwd": {"ms": round(ms_fwd, 4), "tflops": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2)},
+        "bwd": {"ms": round(ms_bwd, 4), "tflops": round(bwd_flops / (ms_bwd * 1e-3) / 1e12, 2)},
+        "roofline": {
+            "kernel": "attn_bwd_dkdv_kernel<128,128,non-causal> (S, dP, dV, dK of one ring step)",
+            "bound": "mfma", "achieved": round(dkdv_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+            "ms_per_launch": round(ms_dkdv, 4),
+        },  # fmt: skip
+        "combine": {
+            "metric": "online_softmax_combine_log2 GB/s ([1,4096,32,128] bf16 x2 -> fp32)",
+            "value": round(comb_gbps, 1), "unit": "GB/s", "us_per_launch": round(ms_comb * 1e3, 2),
+            "bytes": comb_bytes,
+            "roofline": {"bound": "hbm", "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(comb_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+            "cpu_baseline": combine_cpu,
+        },  # fmt: skip
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -152,10 +152,20 @@ typedef struct {
   int32_t causal;
   int32_t dq_dtype, dkv_dtype;
   int32_t accumulate_dq, accumulate_dkv;
+  void* workspace;         /* optional device scratch for pith_attn_bwd_dkdv, 16-byte aligned; may be NULL */
+  int64_t workspace_bytes; /* its size */
 } pith_attn_bwd_args;
 
 int pith_attn_bwd_dkdv(const pith_attn_bwd_args* args, pith_stream_t stream);
 int pith_attn_bwd_dq(const pith_attn_bwd_args* args, pith_stream_t stream);
+
+/* Scratch size with which pith_attn_bwd_dkdv runs fastest for these shapes (0 = none needed).
+ * With grouped-query attention and few key rows the kernel spreads the query heads of a group
+ * over several workgroups, which leave fp32 partial dK/dV in the workspace; a second kernel adds
+ * them in a fixed order (results do not depend on scheduling). Without a workspace, or with a
+ * smaller one, the call still succeeds and one workgroup walks all heads of a group. The
+ * workspace is only used during the call's kernels; nothing is kept in it between calls. */
+int64_t pith_attn_bwd_dkdv_workspace_bytes(const pith_attn_bwd_args* args);
 
 /* ------------------------------------------------------------------------------------------
  * dst[i] = bf16(src[i]) with round-to-nearest-even, i < n. Replaces the reference's

@@ -1,0 +1,59 @@
+// Declarations shared by the two backward kernels (dQ and dK/dV).
+#pragma once
+
+#include "attn_tiles.h"
+
+namespace pith {
+
+struct BwdParams {
+  const __bf16* q;
+  const __bf16* k;
+  const __bf16* v;
+  const __bf16* dout;
+  const float* lse;
+  const float* delta;
+  void* dq;
+  void* dk;
+  void* dv;
+  int Sq, Skv, Hq, Hkv, group, B;
+  int tiles;  // query tiles (dQ kernel) or key tiles (dK/dV kernel) in the grid's x dimension
+  int64_t q_bs, k_bs, v_bs, dout_bs, dq_bs, dk_bs, dv_bs, lse_bs, lse_hs;
+  float kappa, scale;
+  int accumulate;
+  int split;        // dK/dV kernel: query-head groups are cut into `split` parts handled by different workgroups
+  float* ws_dk;     // dK/dV kernel, split > 1: fp32 partial results [split][B][Skv][Hkv][D]
+  float* ws_dv;
+};
+
+// Stores 4 consecutive output features held by one lane; OutT is __bf16 or float.
+template <typename OutT>
+__device__ __forceinline__ void store4(OutT* dst, float a0, float a1, float a2, float a3, bool accumulate);
+
+template <>
+__device__ __forceinline__ void store4<float>(float* dst, float a0, float a1, float a2, float a3, bool accumulate) {
+  f32x4 r = {a0, a1, a2, a3};
+  if (accumulate) r += *reinterpret_cast<const f32x4*>(dst);
+  *reinterpret_cast<f32x4*>(dst) = r;
+}
+
+template <>
+__device__ __forceinline__ void store4<__bf16>(__bf16* dst, float a0, float a1, float a2, float a3, bool accumulate) {
+  if (accumulate) {
+    const u32x2 old = *reinterpret_cast<const u32x2*>(dst);
+    a0 += bf16lo_to_f32(old[0]);
+    a1 += bf16hi_to_f32(old[0]);
+    a2 += bf16lo_to_f32(old[1]);
+    a3 += bf16hi_to_f32(old[1]);
+  }
+  u32x2 w;
+  w[0] = pack_bf16x2(a0, a1);
+  w[1] = pack_bf16x2(a2, a3);
+  *reinterpret_cast<u32x2*>(dst) = w;
+}
+
+
+// Argument checks common to both entry points; returns PITH_OK or records the error.
+int validate_bwd(const pith_attn_bwd_args* a, const char* who, bool need_dq, bool need_dkv);
+BwdParams make_bwd_params(const pith_attn_bwd_args* a);
+
+}  // namespace pith

@@ -1,0 +1,352 @@
+// Key/value-gradient kernel of one chunk attention backward for gfx950, against an external
+// (ring-combined) base-2 LSE and delta = rowsum(O*dO). Follows
+// pithtrain/operators/mla/triton.py:130-197 (non-causal :331-384): P = exp2(kappa*s - lse2) in
+// fp32, masked entries 0, P rounded to bf16 for dV += P^T dO, dS = P*(dP - delta)*scale rounded
+// to bf16 for dK += dS^T Q, fp32 accumulation.
+//
+// Work split. A workgroup of 8 wavefronts owns 128 key rows of one (batch, kv head) and loops
+// over query tiles of 32 rows of the query heads assigned to it. The 8 wavefronts form 4 PAIRS,
+// one per 32 key rows; the two waves of a pair share a SIMD and split the work so that each
+// stays below 256 registers (two waves per SIMD, no accumulator spills):
+//     wave A:  S = Q K^T  ->  P = exp2(kappa*S - lse)  ->  dV^T += dO^T P      (holds K, dV)
+//     wave B:  dP = dO V^T ->  dS = P o (dP - delta) * scale -> dK^T += Q^T dS (holds V, dK)
+// B needs A's P: A leaves the fp32 P tile (32 x 32) in an LDS exchange buffer, in the lane order
+// both waves share, and B picks it up after the iteration's only barrier. Both waves issue the
+// same number of MFMAs (also for 192/128 head dims: 12 + 8 against 8 + 12).
+// The stationary side (K or V rows) sits in registers as B operands, so score tiles have the key
+// index as their column; P / dS then feed the products that contract over queries straight from
+// registers (slot order, see attn_tiles.h) with dO^T / Q^T read transposed from LDS.
+//
+// Query tiles stream through a 3-deep LDS ring: the tile for iteration i+1 is committed while
+// iteration i computes and becomes visible at iteration i's barrier, its buffer having been
+// released by the previous barrier. Global loads run two tiles ahead.
+//
+// With grouped-query attention the heads of a group may be cut into `split` parts handled by
+// different workgroups (more parallelism when there are few key tiles); the parts leave fp32
+// partial results in a caller-provided workspace and a second kernel adds them in a fixed
+// order, so the result does not depend on scheduling.
+#include "attn_bwd_common.h"
+
+namespace pith {
+namespace {
+
+constexpr int kThreads = 512;
+constexpr int kBM = 32;    // query rows per tile
+constexpr int kBN = 128;   // key rows per workgroup
+constexpr int kStages = 3;
+
+template <int DQK, int DV>
+struct DkdvLayout {
+  static constexpr int QP = DQK * 2 + 80;  // tiles are read straight by one wave of a pair, transposed by the other
+  static constexpr int OP = DV * 2 + 80;
+  static constexpr int kQTile = kBM * QP;
+  static constexpr int kOTile = kBM * OP;
+  static constexpr int kStat = 2 * kBM * 4;  // lse[32], delta[32]
+  static constexpr int kStage = kQTile + kOTile + kStat;
+  static constexpr int kExch = 4 * 2 * 4096;  // [pair][parity][32 x 32 fp32]
+  static constexpr int kTotal = kStages * kStage + kExch;
+};
+
+// One wave's loop. ROLE_B = false: wave A (T1 = Q tile, stationary K, out dV). ROLE_B = true:
+// wave B (T1 = dO tile, stationary V, out dK). KDIM = contraction length of the score-type
+// product, ODIM = feature length of the gradient this wave accumulates.
+template <int DQK, int DV, bool CAUSAL, bool ROLE_B, typename Fetch, typename Commit>
+__device__ __forceinline__ void dkdv_wave_loop(const BwdParams& p, char* smem, int lane, int pair, int kv_pair0, int n_iter,
+                                               int n_m, int m_start_wg, const bf16x8* stat,
+                                               f32x16* acc, Fetch& fetch, Commit& commit) {
+  using L = DkdvLayout<DQK, DV>;
+  constexpr int KDIM = ROLE_B ? DV : DQK;
+  constexpr int ODIM = ROLE_B ? DQK : DV;
+  constexpr int T1P = ROLE_B ? L::OP : L::QP;   // pitch of the tile read straight
+  constexpr int T2P = ROLE_B ? L::QP : L::OP;   // pitch of the tile read transposed
+  constexpr int T1_OFF = ROLE_B ? L::kQTile : 0;
+  constexpr int T2_OFF = ROLE_B ? 0 : L::kQTile;
+  const int c = lane & 31, g = lane >> 5;
+  const int key = kv_pair0 + c;
+  const int m_start_pair = CAUSAL ? kv_pair0 / kBM : 0;
+  char* exch = smem + kStages * L::kStage + pair * 8192;
+
+  for (int i = 0; i < n_iter; ++i) {
+    if (i + 1 < n_iter) commit((i + 1) % kStages);
+    if (i + 2 < n_iter) fetch(i + 2);
+    const char* stage = smem + (i % kStages) * L::kStage;
+    const float* stats = reinterpret_cast<const float*>(stage + L::kQTile + L::kOTile);
+    const int mt = m_start_wg + i % n_m;
+    const bool active = mt >= m_start_pair;
+    const int q0 = mt * kBM;
+
+    f32x16 x;
+    bf16x8 frag[2];
+    if (active) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x[v] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KDIM / 16; ++ks) {
+        const bf16x8 a = lds_read_straight(stage + T1_OFF, T1P, c, ks * 16 + g * 8);
+        x = mfma32(a, stat[ks], x);
+      }
+      if (!ROLE_B) {
+        // rows of the tile are queries q0 + acc_row(v, g); this lane's column is `key`
+        const bool masked = (CAUSAL && mt == m_start_pair) || (q0 + kBM > p.Sq);
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          const int r0 = 8 * b4 + 4 * g;
+          const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + r0);
+          f32x4 pr;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float t = __builtin_amdgcn_exp2f(x[4 * b4 + e] * p.kappa - l4[e]);
+            if (masked) {
+              const int qrow = q0 + r0 + e;
+              if ((CAUSAL && key > qrow) || qrow >= p.Sq) t = 0.f;
+            }
+            pr[e] = t;
+            x[4 * b4 + e] = t;
+          }
+          *reinterpret_cast<f32x4*>(exch + (i & 1) * 4096 + (b4 * 64 + lane) * 16) = pr;
+        }
+      }
+    }
+    __syncthreads();
+    if (active) {
+      if (ROLE_B) {
+        const float* delta_s = stats + kBM;
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          const int r0 = 8 * b4 + 4 * g;
+          const f32x4 pr = *reinterpret_cast<const f32x4*>(exch + (i & 1) * 4096 + (b4 * 64 + lane) * 16);
+          const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_s + r0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) x[4 * b4 + e] = pr[e] * (x[4 * b4 + e] - d4[e]) * p.scale;
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+        frag[jj] = to_bf16x8(x[8 * jj], x[8 * jj + 1], x[8 * jj + 2], x[8 * jj + 3], x[8 * jj + 4], x[8 * jj + 5],
+                             x[8 * jj + 6], x[8 * jj + 7]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int o = 0; o < ODIM / 32; ++o) {
+          const bf16x8 a = lds_read_transposed(stage + T2_OFF, T2P, 16 * j, 32 * o, lane);
+          acc[o] = mfma32(a, frag[j], acc[o]);
+        }
+    }
+  }
+}
+
+template <int DQK, int DV, bool CAUSAL, typename OutT>
+__global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
+  using L = DkdvLayout<DQK, DV>;
+  constexpr int KS = DQK / 16, VS = DV / 16, DB = DQK / 32, DVB = DV / 32;
+  constexpr int NSTAT = KS > VS ? KS : VS, NACC = DB > DVB ? DB : DVB;
+  __shared__ __attribute__((aligned(16))) char smem[L::kTotal];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, g = lane >> 5;
+  const int pair = wave & 3;
+  const bool role_b = wave >= 4;
+
+  // linear block id -> (key tile, kv head, batch, head part); early key tiles first: under the
+  // causal mask they see the most query tiles
+  const int per_level = p.Hkv * p.B * p.split;
+  const int n_tile = blockIdx.x / per_level;
+  int pos = blockIdx.x - n_tile * per_level;
+  const int part = pos % p.split;
+  pos /= p.split;
+  const int hk = pos % p.Hkv, b = pos / p.Hkv;
+  const int heads_per_part = p.group / p.split;
+  const int hq0 = hk * p.group + part * heads_per_part;
+
+  const int kv_wg0 = n_tile * kBN;
+  const int kv_pair0 = kv_wg0 + pair * 32;
+  const int key = kv_pair0 + c;
+
+  const int64_t q_row_stride = (int64_t)p.Hq * DQK;
+  const int64_t do_row_stride = (int64_t)p.Hq * DV;
+  const int64_t k_row_stride = (int64_t)p.Hkv * DQK;
+  const int64_t v_row_stride = (int64_t)p.Hkv * DV;
+
+  // stationary fragments: K rows for wave A, V rows for wave B
+  bf16x8 stat[NSTAT];
+  {
+    const int row = key < p.Skv ? key : p.Skv - 1;
+    if (!role_b) {
+      const __bf16* src = p.k + b * p.k_bs + row * k_row_stride + (int64_t)hk * DQK + g * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) stat[ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
+    } else {
+      const __bf16* src = p.v + b * p.v_bs + row * v_row_stride + (int64_t)hk * DV + g * 8;
+#pragma unroll
+      for (int ks = 0; ks < VS; ++ks) stat[ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
+    }
+  }
+  f32x16 acc[NACC];
+#pragma unroll
+  for (int i = 0; i < NACC; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+
+  // Query tiles to visit: all of them, or from the diagonal down under the causal mask.
+  const int m_tiles_all = (p.Sq + kBM - 1) / kBM;
+  const int m_start_wg = CAUSAL ? min(kv_wg0 / kBM, m_tiles_all) : 0;
+  const int n_m = m_tiles_all - m_start_wg;
+  const int n_iter = n_m * heads_per_part;
+
+  TileCopy<kBM, DQK, L::QP, kThreads> qcopy;
+  TileCopy<kBM, DV, L::OP, kThreads> ocopy;
+  float stat_val = 0.f;  // threads 0..31 carry lse, 32..63 carry delta of the tile's rows
+  auto fetch = [&](int it) {
+    const int hq = hq0 + it / n_m;
+    const int mt = m_start_wg + it % n_m;
+    qcopy.fetch(p.q + b * p.q_bs + (int64_t)hq * DQK, q_row_stride, mt * kBM, p.Sq, tid);
+    ocopy.fetch(p.dout + b * p.dout_bs + (int64_t)hq * DV, do_row_stride, mt * kBM, p.Sq, tid);
+    if (tid < 2 * kBM) {
+      int row = mt * kBM + (tid & (kBM - 1));
+      row = row < p.Sq ? row : p.Sq - 1;
+      const float* src = (tid < kBM ? p.lse : p.delta) + b * p.lse_bs + (int64_t)hq * p.lse_hs;
+      stat_val = src[row];
+    }
+  };
+  auto commit = [&](int stage) {
+    char* base = smem + stage * L::kStage;
+    qcopy.commit(base, tid);
+    ocopy.commit(base + L::kQTile, tid);
+    if (tid < 2 * kBM) reinterpret_cast<float*>(base + L::kQTile + L::kOTile)[tid] = stat_val;
+  };
+
+  if (n_iter > 0) {
+    fetch(0);
+    commit(0);
+    if (n_iter > 1) fetch(1);
+  }
+  wait_all_vector_loads();
+  __syncthreads();
+
+  if (!role_b)
+    dkdv_wave_loop<DQK, DV, CAUSAL, false>(p, smem, lane, pair, kv_pair0, n_iter, n_m, m_start_wg, stat, acc, fetch, commit);
+  else
+    dkdv_wave_loop<DQK, DV, CAUSAL, true>(p, smem, lane, pair, kv_pair0, n_iter, n_m, m_start_wg, stat, acc, fetch, commit);
+
+  // ---- epilogue: wave A stores dV, wave B stores dK, for key row `key`, features 32*o + 8*b4 + 4*g ..+3
+  if (key < p.Skv) {
+    const int d = role_b ? DQK : DV;
+    const int nblk = role_b ? DB : DVB;
+    const int64_t row_stride = role_b ? k_row_stride : v_row_stride;
+    if (p.split > 1) {
+      float* ws = (role_b ? p.ws_dk : p.ws_dv) +
+                  (((int64_t)part * p.B + b) * p.Skv + key) * row_stride + (int64_t)hk * d;
+#pragma unroll
+      for (int o = 0; o < NACC; ++o)
+        if (o < nblk)
+#pragma unroll
+          for (int b4 = 0; b4 < 4; ++b4)
+            store4<float>(ws + 32 * o + 8 * b4 + 4 * g, acc[o][4 * b4], acc[o][4 * b4 + 1], acc[o][4 * b4 + 2],
+                          acc[o][4 * b4 + 3], false);
+    } else {
+      OutT* out = reinterpret_cast<OutT*>(role_b ? p.dk : p.dv) + b * (role_b ? p.dk_bs : p.dv_bs) + key * row_stride +
+                  (int64_t)hk * d;
+#pragma unroll
+      for (int o = 0; o < NACC; ++o)
+        if (o < nblk)
+#pragma unroll
+          for (int b4 = 0; b4 < 4; ++b4)
+            store4<OutT>(out + 32 * o + 8 * b4 + 4 * g, acc[o][4 * b4], acc[o][4 * b4 + 1], acc[o][4 * b4 + 2],
+                         acc[o][4 * b4 + 3], p.accumulate != 0);
+    }
+  }
+}
+
+// out[b, s, h, :] (+)= sum over parts of ws[part][b][s][h][:], parts added in index order.
+template <typename OutT>
+__global__ __launch_bounds__(256) void reduce_parts_kernel(const float* __restrict__ ws, OutT* out, int parts,
+                                                           int64_t part_stride, int64_t row_elems, int64_t rows_per_batch,
+                                                           int64_t out_bs, int64_t n4, int accumulate) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t e = i * 4;
+    f32x4 s = *reinterpret_cast<const f32x4*>(ws + e);
+    for (int pidx = 1; pidx < parts; ++pidx) s += *reinterpret_cast<const f32x4*>(ws + pidx * part_stride + e);
+    const int64_t per_batch = rows_per_batch * row_elems;
+    const int64_t bb = e / per_batch;
+    OutT* dst = out + bb * out_bs + (e - bb * per_batch);
+    store4<OutT>(dst, s[0], s[1], s[2], s[3], accumulate != 0);
+  }
+}
+
+int pick_split(const pith_attn_bwd_args* a) {
+  const int64_t group = a->Hq / a->Hkv;
+  const int64_t base = ((a->Skv + kBN - 1) / kBN) * a->Hkv * a->B;
+  int split = 1;
+  while (split < group && base * split < 512 && group % (split * 2) == 0) split *= 2;
+  return split;
+}
+
+int64_t workspace_bytes_for(const pith_attn_bwd_args* a, int split) {
+  if (split <= 1) return 0;
+  return (int64_t)split * a->B * a->Skv * a->Hkv * (a->Dqk + a->Dv) * (int64_t)sizeof(float);
+}
+
+template <int DQK, int DV>
+void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
+  p.tiles = (int)((a->Skv + kBN - 1) / kBN);
+  p.accumulate = a->accumulate_dkv;
+  const dim3 grid((unsigned)(p.tiles * a->Hkv * a->B * p.split)), block(kThreads);
+  const bool f32 = a->dkv_dtype == PITH_F32;
+  if (a->causal) {
+    if (f32) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, true, float>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, true, __bf16>), grid, block, 0, st, p);
+  } else {
+    if (f32) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, false, float>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, false, __bf16>), grid, block, 0, st, p);
+  }
+  if (p.split > 1) {
+    const int64_t rows = a->Skv;
+    for (int which = 0; which < 2; ++which) {
+      const int64_t d = which == 0 ? a->Dqk : a->Dv;
+      const int64_t row_elems = a->Hkv * d;
+      const int64_t part_stride = a->B * rows * row_elems;
+      const int64_t n4 = part_stride / 4;
+      const float* ws = which == 0 ? p.ws_dk : p.ws_dv;
+      void* out = which == 0 ? a->dk : a->dv;
+      const int64_t out_bs = which == 0 ? a->dk_bs : a->dv_bs;
+      const unsigned blocks = (unsigned)((n4 + 255) / 256 < 8192 ? (n4 + 255) / 256 : 8192);
+      if (f32)
+        hipLaunchKernelGGL((reduce_parts_kernel<float>), dim3(blocks), dim3(256), 0, st, ws, (float*)out, p.split,
+                           part_stride, row_elems, rows, out_bs, n4, a->accumulate_dkv);
+      else
+        hipLaunchKernelGGL((reduce_parts_kernel<__bf16>), dim3(blocks), dim3(256), 0, st, ws, (__bf16*)out, p.split,
+                           part_stride, row_elems, rows, out_bs, n4, a->accumulate_dkv);
+    }
+  }
+}
+
+}  // namespace
+}  // namespace pith
+
+using namespace pith;
+
+extern "C" int64_t pith_attn_bwd_dkdv_workspace_bytes(const pith_attn_bwd_args* a) {
+  if (!a || a->Hkv <= 0 || a->Hq <= 0 || a->Hq % a->Hkv != 0 || a->B <= 0 || a->Skv <= 0) return 0;
+  return workspace_bytes_for(a, pick_split(a));
+}
+
+extern "C" int pith_attn_bwd_dkdv(const pith_attn_bwd_args* a, pith_stream_t stream) {
+  const int rc = validate_bwd(a, "pith_attn_bwd_dkdv", false, true);
+  if (rc != PITH_OK) return rc;
+  BwdParams p = make_bwd_params(a);
+  // Head groups are split only when the caller brought a workspace that is large enough.
+  const int split = pick_split(a);
+  const int64_t need = workspace_bytes_for(a, split);
+  if (split > 1 && a->workspace && a->workspace_bytes >= need) {
+    if (!aligned16(a->workspace)) return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_dkdv: workspace must be 16-byte aligned");
+    p.split = split;
+    p.ws_dk = reinterpret_cast<float*>(a->workspace);
+    p.ws_dv = p.ws_dk + (int64_t)split * a->B * a->Skv * a->Hkv * a->Dqk;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (a->Dqk == 128) launch_dkdv<128, 128>(p, a, st);
+  else if (a->Dqk == 192) launch_dkdv<192, 128>(p, a, st);
+  else launch_dkdv<64, 64>(p, a, st);
+  return check_launch("pith_attn_bwd_dkdv");
+}

@@ -2,23 +2,25 @@
 // Numerics follow pithtrain/operators/mla/triton.py:32-93 (causal) and :274-323 (non-causal):
 // fp32 scores from bf16 MFMA, P = exp2(kappa*(s - m)) in fp32, row sum from the fp32 P, P rounded
 // to bf16 for P V, O = acc / l rounded to bf16, LSE2 = log2(l) + kappa*m, kappa = scale*log2(e).
+// One deviation in rounding only: the running maximum m is refreshed (and O, l rescaled) only when
+// a row's tile maximum exceeds it by more than 2^8 in the exp2 domain; P, l and O stay consistent
+// with whichever m is in force, so O and LSE2 are the same function of the inputs.
 //
-// Work split: a workgroup of 4 wavefronts owns 256 consecutive query rows of one (batch, head);
-// each wavefront owns 64 of them (two 32-wide column blocks). K/V tiles of 64 keys are staged
-// through LDS (double buffered, fetched to registers one tile ahead) and shared by the 4 waves.
-// Scores are produced TRANSPOSED, S^T = K Q^T, so that a lane holds one query column: the
-// softmax row reductions are in-lane plus one exchange with the partner lane, and P^T feeds the
-// second product O^T += V^T P^T straight from registers; V^T comes from transposing LDS reads.
+// Work split: a workgroup of WAVES wavefronts owns WAVES*32*QB consecutive query rows of one
+// (batch, head); each wavefront owns 32*QB of them. With QB = 1 a wavefront needs fewer than 256
+// registers, so two wavefronts share a SIMD and one's softmax (VALU) overlaps the other's MFMAs.
+// K/V tiles of 64 keys are staged through LDS (double buffered, fetched to registers one tile
+// ahead) and shared by all waves. Scores are produced TRANSPOSED, S^T = K Q^T, so that a lane
+// holds one query column: the softmax row reductions are in-lane plus one exchange with the
+// partner lane, and P^T feeds the second product O^T += V^T P^T straight from registers; V^T
+// comes from transposing LDS reads.
 #include "attn_tiles.h"
 
 namespace pith {
 namespace {
 
-constexpr int kFwdThreads = 256;
-constexpr int kFwdWaves = 4;
-constexpr int kFwdRowsPerWave = 64;
-constexpr int kFwdBlockM = kFwdWaves * kFwdRowsPerWave;
 constexpr int kFwdBlockN = 64;
+constexpr float kRescaleThreshold = 8.f;  // log2 units
 
 struct FwdParams {
   const __bf16* q;
@@ -27,32 +29,34 @@ struct FwdParams {
   __bf16* o;
   float* lse;
   int Sq, Skv, Hq, Hkv, group;  // group = Hq / Hkv
-  int m_tiles;
+  int B, m_tiles;
   int64_t q_bs, k_bs, v_bs, o_bs, lse_bs, lse_hs;
   float kappa;  // scale * log2(e)
 };
 
-template <int DQK, int DV, bool CAUSAL>
-__global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_fwd_kernel(
-    FwdParams p) {
+template <int DQK, int DV, bool CAUSAL, int QB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void attn_fwd_kernel(FwdParams p) {
+  constexpr int THREADS = WAVES * 64;
+  constexpr int ROWS_WAVE = 32 * QB;
+  constexpr int BM = WAVES * ROWS_WAVE;
+  constexpr int BN = kFwdBlockN;
   constexpr int KS = DQK / 16;         // contraction steps of Q K^T
   constexpr int DVB = DV / 32;         // 32-row blocks of O^T
   constexpr int KP = DQK * 2 + 16;     // K tile pitch: conflict-free 16-byte row reads
   constexpr int VP = DV * 2 + 64;      // V tile pitch: conflict-free transposing reads
-  constexpr int kKTile = kFwdBlockN * KP;
-  constexpr int kVTile = kFwdBlockN * VP;
+  constexpr int kKTile = BN * KP;
+  constexpr int kVTile = BN * VP;
   __shared__ __attribute__((aligned(16))) char smem[2 * (kKTile + kVTile)];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int c = lane & 31, g = lane >> 5;
 
-  // Heaviest (latest) query tiles are scheduled first under the causal mask.
-  const int m_tile = p.m_tiles - 1 - blockIdx.x;
-  const int h = blockIdx.y, b = blockIdx.z;
+  int m_tile, h, b;
+  decode_block(blockIdx.x, p.Hq, p.B, p.m_tiles, m_tile, h, b);
   const int hk = h / p.group;
-  const int m0 = m_tile * kFwdBlockM;
-  const int q_wave0 = m0 + wave * kFwdRowsPerWave;
+  const int m0 = m_tile * BM;
+  const int q_wave0 = m0 + wave * ROWS_WAVE;
 
   const int64_t q_row_stride = (int64_t)p.Hq * DQK;
   const int64_t k_row_stride = (int64_t)p.Hkv * DQK;
@@ -63,9 +67,9 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
   const __bf16* vh = p.v + b * p.v_bs + (int64_t)hk * DV;
 
   // Q^T fragments (B operand): column = query row, slots = 8 consecutive features.
-  bf16x8 qf[2][KS];
+  bf16x8 qf[QB][KS];
 #pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
+  for (int qb = 0; qb < QB; ++qb) {
     int row = q_wave0 + qb * 32 + c;
     row = row < p.Sq ? row : p.Sq - 1;
     const __bf16* src = qh + row * q_row_stride + g * 8;
@@ -73,30 +77,35 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
     for (int ks = 0; ks < KS; ++ks) qf[qb][ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
   }
 
-  f32x16 oacc[DVB][2];
+  f32x16 oacc[DVB][QB];
 #pragma unroll
   for (int i = 0; i < DVB; ++i)
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
+    for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) oacc[i][qb][v] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY};
-  float l_run[2] = {0.f, 0.f};  // this lane's share of the row sum (partner lane holds the rest)
-
-  // Number of key tiles this workgroup / this wavefront has to visit.
-  const int n_tiles_all = (p.Skv + kFwdBlockN - 1) / kFwdBlockN;
-  int n_tiles_wg = n_tiles_all, n_tiles_wave = n_tiles_all;
-  if (CAUSAL) {
-    n_tiles_wg = min(n_tiles_all, (m0 + kFwdBlockM) / kFwdBlockN);
-    n_tiles_wave = min(n_tiles_all, q_wave0 / kFwdBlockN + 1);
+  float m_run[QB], l_run[QB];  // l_run: this lane's share of the row sum (partner lane holds the rest)
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m_run[qb] = -INFINITY;
+    l_run[qb] = 0.f;
   }
 
-  TileCopy<kFwdBlockN, DQK, KP, kFwdThreads> kcopy;
-  TileCopy<kFwdBlockN, DV, VP, kFwdThreads> vcopy;
+  // Number of key tiles this workgroup / this wavefront has to visit.
+  const int n_tiles_all = (p.Skv + BN - 1) / BN;
+  int n_tiles_wg = n_tiles_all, n_tiles_wave = n_tiles_all;
+  if (CAUSAL) {
+    n_tiles_wg = min(n_tiles_all, (m0 + BM - 1) / BN + 1);
+    n_tiles_wave = min(n_tiles_all, (q_wave0 + ROWS_WAVE - 1) / BN + 1);
+  }
+
+  TileCopy<BN, DQK, KP, THREADS> kcopy;
+  TileCopy<BN, DV, VP, THREADS> vcopy;
   kcopy.fetch(kh, k_row_stride, 0, p.Skv, tid);
   vcopy.fetch(vh, v_row_stride, 0, p.Skv, tid);
   kcopy.commit(smem, tid);
   vcopy.commit(smem + kKTile, tid);
+  wait_all_vector_loads();
   __syncthreads();
 
   for (int t = 0; t < n_tiles_wg; ++t) {
@@ -104,17 +113,17 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
     const char* vtile = ktile + kKTile;
     const bool have_next = t + 1 < n_tiles_wg;
     if (have_next) {
-      kcopy.fetch(kh, k_row_stride, (t + 1) * kFwdBlockN, p.Skv, tid);
-      vcopy.fetch(vh, v_row_stride, (t + 1) * kFwdBlockN, p.Skv, tid);
+      kcopy.fetch(kh, k_row_stride, (t + 1) * BN, p.Skv, tid);
+      vcopy.fetch(vh, v_row_stride, (t + 1) * BN, p.Skv, tid);
     }
 
     if (t < n_tiles_wave) {
-      // ---- S^T = K Q^T : [64 keys] x [64 queries] as 2 x 2 tiles of 32 x 32
-      f32x16 s[2][2];
+      // ---- S^T = K Q^T : [64 keys] x [32*QB queries] as 2 x QB tiles of 32 x 32
+      f32x16 s[2][QB];
 #pragma unroll
       for (int kvb = 0; kvb < 2; ++kvb)
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
+        for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
           for (int v = 0; v < 16; ++v) s[kvb][qb][v] = 0.f;
 #pragma unroll
@@ -122,18 +131,16 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
 #pragma unroll
         for (int kvb = 0; kvb < 2; ++kvb) {
           const bf16x8 a = lds_read_straight(ktile, KP, kvb * 32 + c, ks * 16 + g * 8);
-          s[kvb][0] = mfma32(a, qf[0][ks], s[kvb][0]);
-          s[kvb][1] = mfma32(a, qf[1][ks], s[kvb][1]);
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) s[kvb][qb] = mfma32(a, qf[qb][ks], s[kvb][qb]);
         }
       }
 
-      // ---- mask (diagonal tile of a causal chunk, or a ragged last tile)
-      const int n0 = t * kFwdBlockN;
-      const bool diag = CAUSAL && (t == n_tiles_wave - 1) && (n0 + kFwdBlockN - 1 > q_wave0);
-      const bool ragged = n0 + kFwdBlockN > p.Skv;
-      if (diag || ragged) {
+      // ---- mask (tiles crossing the diagonal of a causal chunk, or a ragged last tile)
+      const int n0 = t * BN;
+      if ((CAUSAL && (n0 + BN - 1 > q_wave0)) || (n0 + BN > p.Skv)) {
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
+        for (int qb = 0; qb < QB; ++qb) {
           const int qrow = q_wave0 + qb * 32 + c;
           const int limit = CAUSAL ? min(qrow, p.Skv - 1) : p.Skv - 1;  // last visible key
 #pragma unroll
@@ -147,20 +154,37 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
       }
 
       // ---- online softmax, one query column per lane pair
-      bf16x8 pf[2][4];  // P^T as B operand: [query block][contraction step of 16 keys]
+      float mx[QB];
+      bool refresh = false;
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        float mx = s[0][qb][0];
+      for (int qb = 0; qb < QB; ++qb) {
+        float x = s[0][qb][0];
 #pragma unroll
         for (int kvb = 0; kvb < 2; ++kvb)
 #pragma unroll
-          for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kvb][qb][v]);
-        mx = pair_max(mx);
-        const float m_new = fmaxf(m_run[qb], mx);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row with no visible key yet
-        const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_use) * p.kappa);
-        const float mk = m_use * p.kappa;
-        m_run[qb] = m_new;
+          for (int v = 0; v < 16; ++v) x = fmaxf(x, s[kvb][qb][v]);
+        mx[qb] = pair_max(x);
+        refresh |= (mx[qb] - m_run[qb]) * p.kappa > kRescaleThreshold;  // true on the first tile (m = -inf)
+      }
+      if (__builtin_amdgcn_ballot_w64(refresh) != 0) {  // wave-uniform
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          const float m_new = fmaxf(m_run[qb], mx[qb]);
+          // a row with no visible key so far keeps m = -inf; exp2 of (-inf - -inf) is avoided
+          const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * p.kappa);
+          m_run[qb] = m_new;
+          l_run[qb] *= alpha;
+#pragma unroll
+          for (int i = 0; i < DVB; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oacc[i][qb][v] *= alpha;
+        }
+      }
+
+      bf16x8 pf[QB][4];  // P^T as B operand: [query block][contraction step of 16 keys]
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        const float mk = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb] * p.kappa;
         float rs = 0.f;
 #pragma unroll
         for (int kvb = 0; kvb < 2; ++kvb)
@@ -170,11 +194,7 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
             s[kvb][qb][v] = e;
             rs += e;
           }
-        l_run[qb] = l_run[qb] * alpha + rs;
-#pragma unroll
-        for (int i = 0; i < DVB; ++i)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) oacc[i][qb][v] *= alpha;
+        l_run[qb] += rs;
 #pragma unroll
         for (int kvb = 0; kvb < 2; ++kvb)
 #pragma unroll
@@ -191,8 +211,8 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
 #pragma unroll
         for (int i = 0; i < DVB; ++i) {
           const bf16x8 a = lds_read_transposed(vtile, VP, 16 * j, 32 * i, lane);
-          oacc[i][0] = mfma32(a, pf[0][j], oacc[i][0]);
-          oacc[i][1] = mfma32(a, pf[1][j], oacc[i][1]);
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) oacc[i][qb] = mfma32(a, pf[qb][j], oacc[i][qb]);
         }
       }
     }
@@ -209,7 +229,7 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
   __bf16* oh = p.o + b * p.o_bs + (int64_t)h * DV;
   float* lse = p.lse + b * p.lse_bs + (int64_t)h * p.lse_hs;
 #pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
+  for (int qb = 0; qb < QB; ++qb) {
     const int qrow = q_wave0 + qb * 32 + c;
     const float l = pair_sum(l_run[qb]);
     const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -229,12 +249,15 @@ __global__ __launch_bounds__(kFwdThreads) __attribute__((amdgpu_waves_per_eu(1, 
   }
 }
 
-template <int DQK, int DV>
-void launch_fwd(const FwdParams& p, bool causal, dim3 grid, hipStream_t st) {
-  if (causal)
-    hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV, true>), grid, dim3(kFwdThreads), 0, st, p);
+template <int DQK, int DV, int QB, int WAVES>
+void launch_fwd(FwdParams p, const pith_attn_fwd_args* a, hipStream_t st) {
+  constexpr int BM = WAVES * 32 * QB;
+  p.m_tiles = (int)((a->Sq + BM - 1) / BM);
+  const dim3 grid((unsigned)(p.m_tiles * a->Hq * a->B)), block(WAVES * 64);
+  if (a->causal)
+    hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV, true, QB, WAVES>), grid, block, 0, st, p);
   else
-    hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV, false>), grid, dim3(kFwdThreads), 0, st, p);
+    hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV, false, QB, WAVES>), grid, block, 0, st, p);
 }
 
 }  // namespace
@@ -251,10 +274,13 @@ extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) 
   if (a->Hq % a->Hkv != 0)
     return fail(PITH_ERR_BAD_SHAPE, "pith_attn_fwd: Hq=%lld is not a multiple of Hkv=%lld", (long long)a->Hq,
                 (long long)a->Hkv);
+  if (!(a->scale > 0.f) || !(a->scale < INFINITY))
+    return fail(PITH_ERR_BAD_SHAPE, "pith_attn_fwd: scale=%g must be positive and finite", (double)a->scale);
   if (a->causal && a->Sq != a->Skv)
     return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: causal needs Sq == Skv (got %lld, %lld)", (long long)a->Sq,
                 (long long)a->Skv);
-  if (a->Sq > (1 << 24) || a->Skv > (1 << 24) || a->Hq > 65535 || a->B > 65535)
+  if (a->Sq > (1 << 24) || a->Skv > (1 << 24) || a->Hq > 65535 || a->B > 65535 ||
+      ((a->Sq + 63) / 64) * a->Hq * a->B > 0x7fffffffLL)
     return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: sequence, head or batch count beyond the launch grid limits");
   if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->o) || a->q_bs % 8 || a->k_bs % 8 ||
       a->v_bs % 8 || a->o_bs % 8)
@@ -264,14 +290,13 @@ extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) 
   p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v;
   p.o = (__bf16*)a->o; p.lse = a->lse;
   p.Sq = (int)a->Sq; p.Skv = (int)a->Skv; p.Hq = (int)a->Hq; p.Hkv = (int)a->Hkv; p.group = (int)(a->Hq / a->Hkv);
-  p.m_tiles = (int)((a->Sq + kFwdBlockM - 1) / kFwdBlockM);
+  p.B = (int)a->B; p.m_tiles = 0;
   p.q_bs = a->q_bs; p.k_bs = a->k_bs; p.v_bs = a->v_bs; p.o_bs = a->o_bs; p.lse_bs = a->lse_bs; p.lse_hs = a->lse_hs;
   p.kappa = a->scale * 1.44269504088896340736f;
-  const dim3 grid((unsigned)p.m_tiles, (unsigned)a->Hq, (unsigned)a->B);
   hipStream_t st = (hipStream_t)stream;
-  if (a->Dqk == 128 && a->Dv == 128) launch_fwd<128, 128>(p, a->causal != 0, grid, st);
-  else if (a->Dqk == 192 && a->Dv == 128) launch_fwd<192, 128>(p, a->causal != 0, grid, st);
-  else if (a->Dqk == 64 && a->Dv == 64) launch_fwd<64, 64>(p, a->causal != 0, grid, st);
+  if (a->Dqk == 128 && a->Dv == 128) launch_fwd<128, 128, 1, 8>(p, a, st);
+  else if (a->Dqk == 192 && a->Dv == 128) launch_fwd<192, 128, 1, 8>(p, a, st);
+  else if (a->Dqk == 64 && a->Dv == 64) launch_fwd<64, 64, 1, 8>(p, a, st);
   else
     return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: head dims (Dqk=%lld, Dv=%lld) not in {(64,64),(128,128),(192,128)}",
                 (long long)a->Dqk, (long long)a->Dv);

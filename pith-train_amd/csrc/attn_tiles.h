@@ -76,6 +76,30 @@ __device__ __forceinline__ bf16x8 to_bf16x8(float a0, float a1, float a2, float 
   return r;
 }
 
+// Waits until every vector-memory load issued so far has returned. Placed once before a main
+// loop, after the loop-invariant fragments were fetched: otherwise the compiler keeps the waits
+// for those fragments inside the loop, where they also wait for the loads that prefetch the next
+// tile and so expose the global-memory latency in every iteration.
+__device__ __forceinline__ void wait_all_vector_loads() {
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt left at their maxima
+}
+
+// Maps a linear workgroup id to (tile, head, batch) so that
+//   - tiles are visited from `tiles-1` down to 0 across ALL heads (under a causal mask the late
+//     tiles carry the most work, and the lightest workgroups should be the last ones dispatched);
+//   - workgroups are dealt round-robin to the 8 XCDs of the device, each with its own L2: the
+//     heads of one level are permuted so that an XCD keeps a contiguous range of heads, i.e. the
+//     query heads that share a kv head read their K/V through the same L2.
+__device__ __forceinline__ void decode_block(int linear, int heads, int batch, int tiles, int& tile, int& h, int& b) {
+  const int per_level = heads * batch;
+  const int level = linear / per_level;
+  int pos = linear - level * per_level;
+  if ((per_level & 7) == 0) pos = (pos & 7) * (per_level >> 3) + (pos >> 3);
+  tile = tiles - 1 - level;
+  b = pos / heads;
+  h = pos - b * heads;
+}
+
 // Cooperative copy of a [ROWS x COLS] bf16 tile between global memory and LDS by THREADS threads,
 // split into a "fetch to registers" half and a "store to LDS" half so that the global loads of
 // the next tile can be in flight while the current tile is consumed.

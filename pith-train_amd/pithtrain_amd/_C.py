@@ -77,6 +77,7 @@ class AttnBwdArgs(Structure):
         ("scale", c_float), ("causal", c_int32),
         ("dq_dtype", c_int32), ("dkv_dtype", c_int32),
         ("accumulate_dq", c_int32), ("accumulate_dkv", c_int32),
+        ("workspace", c_void_p), ("workspace_bytes", c_int64),
     ]  # fmt: skip
 
 
@@ -90,6 +91,7 @@ SYMBOLS = {
     "pith_attn_bwd_delta": (c_int, [POINTER(AttnDeltaArgs), c_void_p]),
     "pith_attn_bwd_dkdv": (c_int, [POINTER(AttnBwdArgs), c_void_p]),
     "pith_attn_bwd_dq": (c_int, [POINTER(AttnBwdArgs), c_void_p]),
+    "pith_attn_bwd_dkdv_workspace_bytes": (c_int64, [POINTER(AttnBwdArgs)]),
     "pith_cast_f32_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
 }
 

@@ -99,6 +99,7 @@ def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal) -> _C.AttnBwdArg
         dq_bs=0, dk_bs=0, dv_bs=0, lse_bs=lse_bs, lse_hs=lse_hs,
         scale=float(softmax_scale), causal=int(bool(causal)),
         dq_dtype=_C.PITH_BF16, dkv_dtype=_C.PITH_BF16, accumulate_dq=0, accumulate_dkv=0,
+        workspace=None, workspace_bytes=0,
     )  # fmt: skip
 
 
@@ -114,6 +115,13 @@ def attn_bwd_dkdv_into(
     args.dk_bs, args.dv_bs = _C.bshd_batch_stride(dk, "dk"), _C.bshd_batch_stride(dv, "dv")
     args.dkv_dtype = _C.dtype_code(dk)
     args.accumulate_dkv = int(bool(accumulate))
+    # Scratch for the head-split partial sums; the caching allocator makes this a pointer bump,
+    # and stream ordering keeps the block alive until the kernels that use it have run.
+    need = _C.lib().pith_attn_bwd_dkdv_workspace_bytes(_C.byref(args))
+    workspace = None
+    if need > 0:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        args.workspace, args.workspace_bytes = workspace.data_ptr(), need
     _C.check(_C.lib().pith_attn_bwd_dkdv(_C.byref(args), _C.current_stream(q)))
 
 

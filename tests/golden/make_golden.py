@@ -18,8 +18,8 @@ sys.path.insert(0, ROOT)
 from oracle import ring_oracle as R  # noqa: E402
 
 CASES = {  # name: (Hq, Hkv, Dqk, Dv, S_local, C, rank)
-    "gqa": (4, 2, 128, 128, 64, 2, 1),
-    "mla": (2, 2, 192, 128, 64, 2, 0),
+    "gqa": (2, 1, 128, 128, 32, 2, 1),
+    "mla": (1, 1, 192, 128, 32, 2, 0),
 }
 
 

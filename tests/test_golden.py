@@ -11,7 +11,7 @@ from helpers import check_bf16_result, check_lse
 from oracle import ring_oracle as R
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ring_small.npz")
-CASES = {"gqa": (4, 2, 128, 128, 64, 2, 1), "mla": (2, 2, 192, 128, 64, 2, 0)}
+CASES = {"gqa": (2, 1, 128, 128, 32, 2, 1), "mla": (1, 1, 192, 128, 32, 2, 0)}
 
 
 def _load(name):

@@ -261,7 +261,7 @@ extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t strea
   if (rc != PITH_OK) return rc;
   const BwdParams p = make_bwd_params(a);
   hipStream_t st = (hipStream_t)stream;
-  if (a->Dqk == 128) launch_dq<128, 128, 1, 1, 8>(p, a, st);
+  if (a->Dqk == 128) launch_dq<128, 128, 1, 2, 8>(p, a, st);
   else if (a->Dqk == 192) launch_dq<192, 128, 1, 1, 8>(p, a, st);
   else launch_dq<64, 64, 1, 1, 8>(p, a, st);
   return check_launch("pith_attn_bwd_dq");

@@ -14,25 +14,10 @@
 // holds one query column: the softmax row reductions are in-lane plus one exchange with the
 // partner lane, and P^T feeds the second product O^T += V^T P^T straight from registers; V^T
 // comes from transposing LDS reads.
-#include "attn_tiles.h"
+#include "attn_fwd_common.h"
 
 namespace pith {
 namespace {
-
-constexpr int kFwdBlockN = 64;
-constexpr float kRescaleThreshold = 8.f;  // log2 units
-
-struct FwdParams {
-  const __bf16* q;
-  const __bf16* k;
-  const __bf16* v;
-  __bf16* o;
-  float* lse;
-  int Sq, Skv, Hq, Hkv, group;  // group = Hq / Hkv
-  int B, m_tiles;
-  int64_t q_bs, k_bs, v_bs, o_bs, lse_bs, lse_hs;
-  float kappa;  // scale * log2(e)
-};
 
 template <int DQK, int DV, bool CAUSAL, int QB, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void attn_fwd_kernel(FwdParams p) {
@@ -294,7 +279,7 @@ extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) 
   p.q_bs = a->q_bs; p.k_bs = a->k_bs; p.v_bs = a->v_bs; p.o_bs = a->o_bs; p.lse_bs = a->lse_bs; p.lse_hs = a->lse_hs;
   p.kappa = a->scale * 1.44269504088896340736f;
   hipStream_t st = (hipStream_t)stream;
-  if (a->Dqk == 128 && a->Dv == 128) launch_fwd<128, 128, 1, 8>(p, a, st);
+  if (a->Dqk == 128 && a->Dv == 128) launch_fwd_d128(p, a->causal != 0, st);
   else if (a->Dqk == 192 && a->Dv == 128) launch_fwd<192, 128, 1, 8>(p, a, st);
   else if (a->Dqk == 64 && a->Dv == 64) launch_fwd<64, 64, 1, 8>(p, a, st);
   else

@@ -1,0 +1,26 @@
+// Declarations shared by the forward kernels.
+#pragma once
+
+#include "attn_tiles.h"
+
+namespace pith {
+
+constexpr int kFwdBlockN = 64;            // keys per LDS tile
+constexpr float kRescaleThreshold = 8.f;  // log2 units, see attn_fwd.hip
+
+struct FwdParams {
+  const __bf16* q;
+  const __bf16* k;
+  const __bf16* v;
+  __bf16* o;
+  float* lse;
+  int Sq, Skv, Hq, Hkv, group;  // group = Hq / Hkv
+  int B, m_tiles;
+  int64_t q_bs, k_bs, v_bs, o_bs, lse_bs, lse_hs;
+  float kappa;  // scale * log2(e)
+};
+
+// Forward for head dims (128, 128): attn_fwd_d128.hip.
+void launch_fwd_d128(FwdParams p, bool causal, hipStream_t stream);
+
+}  // namespace pith

@@ -137,4 +137,100 @@ struct TileCopy {
   }
 };
 
+// ---------------------------------------------------------------------------------------------
+// 128-feature tiles moved global memory -> LDS directly (global_load_lds_dwordx4), without
+// passing through registers. One wavefront instruction moves 64 pieces of 16 bytes to 1 KB of
+// consecutive LDS (lane L -> byte 16*L of the region), so tile rows are packed at 256 bytes
+// (16 pieces) with no padding; bank conflicts are avoided by keeping piece q of row r at
+// position q ^ tile_swizzle(r). The swizzle is a bijection of r % 16 (16 consecutive rows read
+// "straight" at one feature offset hit 16 different positions) and moves rows r..r+3 to four
+// different 64-byte groups (what the transposing read touches at once).
+constexpr int kRowBytes128 = 256;
+
+__device__ __forceinline__ int tile_swizzle(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
+// Byte offset inside a packed tile of the 16-byte piece `piece` (0..15) of row `row`.
+__device__ __forceinline__ int swizzled_offset(int row, int piece) {
+  return row * kRowBytes128 + ((piece ^ tile_swizzle(row)) << 4);
+}
+
+// 16 bytes per lane from global address `base` + `offset` (base the same for all lanes, offset
+// per lane, unsigned) to LDS at `dst_wave` + 16 * lane; `dst_wave` must be the same for all lanes
+// of the wavefront. Completion is tracked by vmcnt, in issue order with the other vector loads.
+// Written as inline assembly on purpose: the compiler does not see an LDS write, so it places no
+// wait between this load and later LDS reads of OTHER tiles; the caller waits (s_waitcnt vmcnt)
+// and synchronises the workgroup before anyone reads the destination.
+__device__ __forceinline__ void load_lds16(const char* base, int offset, char* dst_wave) {
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char*)dst_wave;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(offset), "s"(base)
+               : "memory");  // m0 is written here and by nothing else in the kernels that use this
+}
+
+// Moves a [ROWS x 128] bf16 tile with THREADS threads (THREADS / 64 wavefronts): wavefront w
+// moves the 4 tile rows of every 1 KB region n * WAVES + w.
+template <int ROWS, int THREADS>
+struct DirectTile128 {
+  static constexpr int kWaves = THREADS / 64;
+  static constexpr int kPerThread = ROWS * 16 / THREADS;
+  static_assert(ROWS * 16 % THREADS == 0, "tile must split evenly over the threads");
+  static constexpr int kTileBytes = ROWS * kRowBytes128;
+  int src_off[kPerThread];  // byte offset of this lane's source piece from the tile's first row
+  int row_bytes;
+
+  // row_bytes: distance between consecutive rows in global memory, in bytes
+  __device__ __forceinline__ void init(int row_bytes_, int wave, int lane) {
+    row_bytes = row_bytes_;
+#pragma unroll
+    for (int n = 0; n < kPerThread; ++n) {
+      const int row = 4 * (n * kWaves + wave) + (lane >> 4);
+      src_off[n] = row * row_bytes + (((lane & 15) ^ tile_swizzle(row)) << 4);
+    }
+  }
+  // tile_src: address of [first row of the tile][feature 0] of the head slice (uniform);
+  // rows_left: valid rows from there on (>= 1), rows beyond are read from the last valid row.
+  // `slot` is the LDS tile (uniform).
+  __device__ __forceinline__ void issue(const char* tile_src, int rows_left, char* slot, int wave, int lane) const {
+    if (rows_left >= ROWS) {
+#pragma unroll
+      for (int n = 0; n < kPerThread; ++n) load_lds16(tile_src, src_off[n], slot + (n * kWaves + wave) * 1024);
+    } else {
+#pragma unroll
+      for (int n = 0; n < kPerThread; ++n) {
+        const int row = 4 * (n * kWaves + wave) + (lane >> 4);
+        const int src_row = row < rows_left ? row : rows_left - 1;
+        load_lds16(tile_src, src_row * row_bytes + (((lane & 15) ^ tile_swizzle(row)) << 4),
+                   slot + (n * kWaves + wave) * 1024);
+      }
+    }
+  }
+};
+
+// Per-lane offsets for reading a packed swizzled tile.
+// straight_offset(c, piece): fragment of row c (+ a multiple of 16 rows added by the caller as
+// rows * 256 bytes), features 8*piece .. 8*piece+7.
+__device__ __forceinline__ int straight_offset128(int row, int piece) { return swizzled_offset(row, piece); }
+
+// Offset for one ds_read_b64_tr_b16 of a transposed fragment (see lds_read_transposed): tile
+// rows row_base + 8*half + 4*(blk>>1) + (r>>2), features col_base + 16*(blk&1) + 4*(r&3) .. +3.
+// row_base must be a multiple of 16, col_base a multiple of 32.
+__device__ __forceinline__ int transposed_offset128(int row_base, int half, int col_base, int lane) {
+  const int r = lane & 15, blk = lane >> 4;
+  const int row = row_base + 8 * half + 4 * (blk >> 1) + (r >> 2);
+  const int col = col_base + 16 * (blk & 1) + 4 * (r & 3);  // features
+  return swizzled_offset(row, col >> 3) + ((col & 7) << 1);
+}
+
+__device__ __forceinline__ bf16x8 lds_read_transposed_at(const char* lo_addr, const char* hi_addr) {
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(lo_addr));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(hi_addr));
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  s16x8 v;
+  v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
+  v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
+  return __builtin_bit_cast(bf16x8, v);
+}
+
 }  // namespace pith

@@ -52,6 +52,11 @@ __device__ __forceinline__ void store4<__bf16>(__bf16* dst, float a0, float a1, 
 }
 
 
+// dK/dV kernels: a workgroup owns kDkdvBlockN key rows (the grid and the head split depend on it).
+constexpr int kDkdvBlockN = 128;
+// dK/dV for head dims (128, 128): attn_bwd_dkdv_d128.hip. p.tiles, p.split, p.ws_* are set by the caller.
+void launch_dkdv_d128(const BwdParams& p, bool causal, bool f32_out, unsigned grid, hipStream_t stream);
+
 // Argument checks common to both entry points; returns PITH_OK or records the error.
 int validate_bwd(const pith_attn_bwd_args* a, const char* who, bool need_dq, bool need_dkv);
 BwdParams make_bwd_params(const pith_attn_bwd_args* a);

@@ -32,7 +32,7 @@ namespace {
 
 constexpr int kThreads = 512;
 constexpr int kBM = 32;    // query rows per tile
-constexpr int kBN = 128;   // key rows per workgroup
+constexpr int kBN = kDkdvBlockN;  // key rows per workgroup
 constexpr int kStages = 3;
 
 template <int DQK, int DV>
@@ -293,12 +293,16 @@ void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
   p.accumulate = a->accumulate_dkv;
   const dim3 grid((unsigned)(p.tiles * a->Hkv * a->B * p.split)), block(kThreads);
   const bool f32 = a->dkv_dtype == PITH_F32;
-  if (a->causal) {
-    if (f32) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, true, float>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, true, __bf16>), grid, block, 0, st, p);
+  if constexpr (DQK == 128 && DV == 128) {
+    launch_dkdv_d128(p, a->causal != 0, f32, grid.x, st);
   } else {
-    if (f32) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, false, float>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, false, __bf16>), grid, block, 0, st, p);
+    if (a->causal) {
+      if (f32) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, true, float>), grid, block, 0, st, p);
+      else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, true, __bf16>), grid, block, 0, st, p);
+    } else {
+      if (f32) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, false, float>), grid, block, 0, st, p);
+      else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, false, __bf16>), grid, block, 0, st, p);
+    }
   }
   if (p.split > 1) {
     const int64_t rows = a->Skv;

@@ -1,0 +1,353 @@
+// Key/value-gradient kernel for head dims (128, 128) on gfx950. Same function and numerics as the
+// general kernel in attn_bwd_dkdv.hip (pithtrain/operators/mla/triton.py:130-197, :331-384:
+// P = exp2(kappa*s - lse2) in fp32, masked entries 0, P rounded to bf16 for dV += P^T dO,
+// dS = P*(dP - delta)*scale rounded to bf16 for dK += dS^T Q, fp32 accumulation), same work split:
+// a workgroup of 8 wavefronts owns 128 key rows of one (batch, kv head) and streams query tiles
+// of its query heads; the wavefronts form 4 pairs, one per 32 keys, wave A of a pair holds K and
+// dV, wave B holds V and dK, and A hands the fp32 P tile to B through an LDS buffer.
+//
+// What differs from the general kernel (all of it measured to matter on the device):
+//   - query tiles are 64 rows, so a wave issues 32 MFMAs between synchronisations;
+//   - Q / dO tiles and the lse / delta rows go global -> LDS directly (global_load_lds) into a
+//     ring of three stages, requested one interval ahead; tiles are packed and swizzled;
+//   - B runs ONE TILE BEHIND A. In interval i wave A computes dV(i-1), S(i), P(i); wave B
+//     computes dS(i-1), dK(i-1), dP(i);
+//   - A runs [matrix block | vector block], B runs [vector block | matrix block], with a
+//     workgroup barrier at "|" and at the end of the interval. The two waves of a pair share a
+//     SIMD, so the matrix pipe is always owned by exactly one of them while the other does its
+//     exp / dS arithmetic, tile requests and bookkeeping. The middle barrier also orders B's read
+//     of P(i-1) before A's write of P(i): one P buffer per pair is enough;
+//   - inside a matrix block the LDS fragment reads run kAhead products ahead of their use.
+#include <type_traits>
+
+#include "attn_bwd_common.h"
+
+namespace pith {
+namespace {
+
+constexpr int kThreads = 512;
+constexpr int kBM = 64;             // query rows per tile
+constexpr int kBN = kDkdvBlockN;    // key rows per workgroup
+constexpr int kD = 128;
+constexpr int kStages = 3;          // tiles i-1, i (in use) and i+1 (landing)
+constexpr int kAhead = 4;           // fragment reads run this many products ahead
+constexpr int kTile = kBM * kRowBytes128;        // 16 KB
+constexpr int kStat = 2 * kBM * 4;               // lse[64], delta[64]
+constexpr int kStage = 2 * kTile + kStat;        // Q tile, dO tile, stats
+constexpr int kExchPair = kBM * 32 * 4;          // one 64 x 32 fp32 P tile
+constexpr int kSmem = kStages * kStage + 4 * kExchPair;
+
+// Position of a query tile in the stream of (query head, tile) pairs a workgroup visits.
+struct TileCursor {
+  int hq, mt;
+  __device__ __forceinline__ void advance(int m_first, int m_end) {
+    if (++mt == m_end) {
+      mt = m_first;
+      ++hq;
+    }
+  }
+};
+
+template <bool CAUSAL, typename OutT>
+__global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams p) {
+  constexpr int KS = kD / 16, DB = kD / 32;
+  __shared__ __attribute__((aligned(1024))) char smem[kSmem];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31, g = lane >> 5;
+  const int pair = wave & 3;
+  const bool role_b = wave >= 4;
+
+  // linear block id -> (key tile, kv head, batch, head part); early key tiles first: under the
+  // causal mask they see the most query tiles
+  const int per_level = p.Hkv * p.B * p.split;
+  const int n_tile = blockIdx.x / per_level;
+  int pos = blockIdx.x - n_tile * per_level;
+  const int part = pos % p.split;
+  pos /= p.split;
+  const int hk = pos % p.Hkv, b = pos / p.Hkv;
+  const int heads_per_part = p.group / p.split;
+  const int hq0 = hk * p.group + part * heads_per_part;
+
+  const int kv_wg0 = n_tile * kBN;
+  const int kv_pair0 = kv_wg0 + pair * 32;
+  const int key = kv_pair0 + c;
+
+  const int q_row_bytes = p.Hq * kD * 2;  // Q and dO rows
+  const int64_t kv_row_stride = (int64_t)p.Hkv * kD;
+
+  // Query tiles to visit: all of them, or from the diagonal down under the causal mask.
+  const int m_end = (p.Sq + kBM - 1) / kBM;
+  const int m_first = CAUSAL ? min(kv_wg0 / kBM, m_end) : 0;
+  const int n_iter = (m_end - m_first) * heads_per_part;
+
+  // ---- requests
+  DirectTile128<kBM, kThreads> mover;
+  mover.init(q_row_bytes, wave, lane);
+  const char* q_base = reinterpret_cast<const char*>(p.q + b * p.q_bs);
+  const char* do_base = reinterpret_cast<const char*>(p.dout + b * p.dout_bs);
+  TileCursor req = {hq0, m_first};
+  auto request = [&](char* stage) __attribute__((always_inline)) {
+    const int row0 = req.mt * kBM;
+    const int64_t head_off = (int64_t)req.hq * kD * 2 + (int64_t)row0 * q_row_bytes;
+    mover.issue(q_base + head_off, p.Sq - row0, stage, wave, lane);
+    mover.issue(do_base + head_off, p.Sq - row0, stage + kTile, wave, lane);
+    if (wave < 2) {  // wave 0 fetches the 64 lse values of the tile's rows, wave 1 the 64 delta values
+      int row = row0 + lane;
+      row = row < p.Sq ? row : p.Sq - 1;
+      const float* src = (wave == 0 ? p.lse : p.delta) + b * p.lse_bs + (int64_t)req.hq * p.lse_hs + row;
+      load_lds4(src, stage + 2 * kTile + wave * kBM * 4);
+    }
+    req.advance(m_first, m_end);
+  };
+  if (n_iter > 0) request(smem);
+
+  // stationary fragments: K rows for wave A, V rows for wave B
+  bf16x8 stat[KS];
+  {
+    const int row = key < p.Skv ? key : p.Skv - 1;
+    const __bf16* src = (role_b ? p.v + b * p.v_bs : p.k + b * p.k_bs) + row * kv_row_stride + (int64_t)hk * kD + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) stat[ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
+  }
+  f32x16 acc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+
+  // per-lane read offsets inside a tile
+  int s_off[KS];     // straight fragment of tile row c, contraction step ks (+ 32 rows: + 8192 bytes)
+  int t_off[DB][2];  // transposing reads of feature block o, lower / upper 8 rows (+ 16 rows: + 4096 bytes)
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) s_off[ks] = straight_offset128(c, 2 * ks + g);
+#pragma unroll
+  for (int o = 0; o < DB; ++o)
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) t_off[o][hh] = transposed_offset128(0, hh, 32 * o, lane);
+
+  // Within a stage wave A reads Q straight and dO transposed, wave B dO straight and Q transposed.
+  const int straight_tile = role_b ? kTile : 0;
+  const int transposed_tile = role_b ? 0 : kTile;
+  char* const exch = smem + kStages * kStage + pair * kExchPair;
+
+  f32x16 x[2];      // [32-row block] A: S, then P of the current tile. B: dP, kept into the next interval
+  bf16x8 frag[4];   // [16-row step] A: P(i) as B operand of dV(i) in the next interval. B: dS(i-1) for dK(i-1)
+
+  // score-type product of the tile in `stage`: x = T1 * stat^T
+  auto straight_product = [&](const char* stage) __attribute__((always_inline)) {
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x[rb][v] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(stage + straight_tile + s_off[ks] + rb * 32 * kRowBytes128);
+        x[rb] = mfma32(a, stat[ks], x[rb]);
+      }
+  };
+  // gradient-type product with the tile in `stage`: acc^T += T2^T * frag
+  auto transposed_product = [&](const char* stage) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int o = 0; o < DB; ++o) {
+        const char* base = stage + transposed_tile + j * 16 * kRowBytes128;
+        const bf16x8 a = lds_read_transposed_at(base + t_off[o][0], base + t_off[o][1]);
+        acc[o] = mfma32(a, frag[j], acc[o]);
+      }
+  };
+  // both (gradient product of `stage_prev`, then score product of `stage_cur`), with the
+  // fragment reads kAhead products ahead
+  auto matrix_block = [&](const char* stage_prev, const char* stage_cur) __attribute__((always_inline)) {
+    constexpr int NT = 4 * DB, NS = 2 * KS;
+    static_assert(kAhead <= NT, "look-ahead assumes it starts inside the gradient product");
+    bf16x8 at[4][DB], as[KS][2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int o = 0; o < DB; ++o) {
+        const char* base = stage_prev + transposed_tile + j * 16 * kRowBytes128;
+        at[j][o] = lds_read_transposed_at(base + t_off[o][0], base + t_off[o][1]);
+      }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+        as[ks][rb] = *reinterpret_cast<const bf16x8*>(stage_cur + straight_tile + s_off[ks] + rb * 32 * kRowBytes128);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int o = 0; o < DB; ++o) acc[o] = mfma32(at[j][o], frag[j], acc[o]);
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x[rb][v] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) x[rb] = mfma32(as[ks][rb], stat[ks], x[rb]);
+    // a transposed fragment takes two LDS reads, a straight one a single read
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+    for (int m = 0; m < NT - kAhead; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+#pragma unroll
+    for (int m = 0; m < NS; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+  };
+
+  // A: x = S of query tile mt -> P, left in the exchange buffer (fp32) and in frag (bf16).
+  // Rows of the tile are queries q0 + 32*rb + acc_row(v, g); this lane's column is `key`.
+  auto make_p = [&](const char* stage, int mt) __attribute__((always_inline)) {
+    const float* lse_s = reinterpret_cast<const float*>(stage + 2 * kTile);
+    const int q0 = mt * kBM;
+    f32x4 l4[2][4];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) l4[rb][b4] = *reinterpret_cast<const f32x4*>(lse_s + 32 * rb + 8 * b4 + 4 * g);
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x[rb][v] = __builtin_amdgcn_exp2f(x[rb][v] * p.kappa - l4[rb][v >> 2][v & 3]);
+    if ((CAUSAL && q0 < kv_pair0 + 31) || (q0 + kBM > p.Sq)) {
+      // tile on the diagonal of a causal chunk, or a ragged last tile (wave-uniform branch)
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int qrow = q0 + 32 * rb + acc_row(v, g);
+          if ((CAUSAL && key > qrow) || qrow >= p.Sq) x[rb][v] = 0.f;
+        }
+    }
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) {
+        const f32x4 pr = {x[rb][4 * b4], x[rb][4 * b4 + 1], x[rb][4 * b4 + 2], x[rb][4 * b4 + 3]};
+        *reinterpret_cast<f32x4*>(exch + ((rb * 4 + b4) * 64 + lane) * 16) = pr;
+      }
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+        frag[2 * rb + jj] = to_bf16x8(x[rb][8 * jj], x[rb][8 * jj + 1], x[rb][8 * jj + 2], x[rb][8 * jj + 3],
+                                      x[rb][8 * jj + 4], x[rb][8 * jj + 5], x[rb][8 * jj + 6], x[rb][8 * jj + 7]);
+    }
+  };
+  // B: x = dP of the tile in `stage`, P from the exchange buffer -> dS in frag (bf16)
+  auto make_ds = [&](const char* stage) __attribute__((always_inline)) {
+    const float* delta_s = reinterpret_cast<const float*>(stage + 2 * kTile) + kBM;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+      f32x4 pr[4], d4[4];
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) {
+        pr[b4] = *reinterpret_cast<const f32x4*>(exch + ((rb * 4 + b4) * 64 + lane) * 16);
+        d4[b4] = *reinterpret_cast<const f32x4*>(delta_s + 32 * rb + 8 * b4 + 4 * g);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x[rb][v] = pr[v >> 2][v & 3] * (x[rb][v] - d4[v >> 2][v & 3]) * p.scale;
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+        frag[2 * rb + jj] = to_bf16x8(x[rb][8 * jj], x[rb][8 * jj + 1], x[rb][8 * jj + 2], x[rb][8 * jj + 3],
+                                      x[rb][8 * jj + 4], x[rb][8 * jj + 5], x[rb][8 * jj + 6], x[rb][8 * jj + 7]);
+    }
+  };
+
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far: tile 0, stationary fragments
+  __syncthreads();
+
+  // Interval i = 0 .. n_iter touches tiles i-1 and i; tile -1 and tile n_iter do not exist.
+  // Ring stages rotate: prev <- cur <- next <- (the stage prev used to be).
+  auto run = [&](auto role_tag) __attribute__((always_inline)) {
+    constexpr bool ROLE_B = decltype(role_tag)::value;
+    TileCursor cur = {hq0, m_first};
+    bool prev_active = false;
+    int off_prev = 2 * kStage, off_cur = 0, off_next = kStage;
+    for (int i = 0; i <= n_iter; ++i) {
+      const char* stage_cur = smem + off_cur;
+      const char* stage_prev = smem + off_prev;
+      const bool have_cur = i < n_iter;
+      // under the causal mask a pair skips the tiles that lie entirely above its diagonal
+      const bool cur_active = have_cur && (!CAUSAL || cur.mt * kBM + kBM > kv_pair0);
+      const bool will_request = i + 1 < n_iter;
+      if (!ROLE_B) {
+        if (prev_active && cur_active) matrix_block(stage_prev, stage_cur);
+        else {
+          if (prev_active) transposed_product(stage_prev);
+          if (cur_active) straight_product(stage_cur);
+        }
+        __syncthreads();  // B has read P(i-1); the matrix pipe passes to B
+        if (will_request) request(smem + off_next);
+        if (cur_active) make_p(stage_cur, cur.mt);
+      } else {
+        if (will_request) request(smem + off_next);
+        if (prev_active) make_ds(stage_prev);
+        __syncthreads();
+        if (prev_active && cur_active) matrix_block(stage_prev, stage_cur);
+        else {
+          if (prev_active) transposed_product(stage_prev);
+          if (cur_active) straight_product(stage_cur);
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // tile i+1 has landed
+      __syncthreads();
+      prev_active = cur_active;
+      if (have_cur) cur.advance(m_first, m_end);
+      const int t = off_prev;
+      off_prev = off_cur;
+      off_cur = off_next;
+      off_next = t;
+    }
+  };
+  // Both roles pass the same barriers; separate loops keep each body straight-line.
+  if (n_iter > 0) {
+    if (!role_b) run(std::false_type{});
+    else run(std::true_type{});
+  }
+
+  // ---- epilogue: wave A stores dV, wave B stores dK, for key row `key`, features 32*o + 8*b4 + 4*g ..+3
+  if (key < p.Skv) {
+    if (p.split > 1) {
+      float* ws = (role_b ? p.ws_dk : p.ws_dv) + (((int64_t)part * p.B + b) * p.Skv + key) * kv_row_stride + (int64_t)hk * kD;
+#pragma unroll
+      for (int o = 0; o < DB; ++o)
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4)
+          store4<float>(ws + 32 * o + 8 * b4 + 4 * g, acc[o][4 * b4], acc[o][4 * b4 + 1], acc[o][4 * b4 + 2],
+                        acc[o][4 * b4 + 3], false);
+    } else {
+      OutT* out = reinterpret_cast<OutT*>(role_b ? p.dk : p.dv) + b * (role_b ? p.dk_bs : p.dv_bs) + key * kv_row_stride +
+                  (int64_t)hk * kD;
+#pragma unroll
+      for (int o = 0; o < DB; ++o)
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4)
+          store4<OutT>(out + 32 * o + 8 * b4 + 4 * g, acc[o][4 * b4], acc[o][4 * b4 + 1], acc[o][4 * b4 + 2],
+                       acc[o][4 * b4 + 3], p.accumulate != 0);
+    }
+  }
+}
+
+}  // namespace
+
+void launch_dkdv_d128(const BwdParams& p, bool causal, bool f32_out, unsigned grid, hipStream_t st) {
+  const dim3 g(grid), block(kThreads);
+  if (causal) {
+    if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, float>), g, block, 0, st, p);
+    else hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, __bf16>), g, block, 0, st, p);
+  } else {
+    if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<false, float>), g, block, 0, st, p);
+    else hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<false, __bf16>), g, block, 0, st, p);
+  }
+}
+
+}  // namespace pith

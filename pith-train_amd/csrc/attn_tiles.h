@@ -168,6 +168,16 @@ __device__ __forceinline__ void load_lds16(const char* base, int offset, char* d
                : "memory");  // m0 is written here and by nothing else in the kernels that use this
 }
 
+// 4 bytes per lane from the per-lane global address `src` to LDS at `dst_wave` + 4 * lane (same
+// conventions as load_lds16).
+__device__ __forceinline__ void load_lds4(const void* src, char* dst_wave) {
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char*)dst_wave;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+               :
+               : "s"(lds_addr), "v"(src)
+               : "memory");
+}
+
 // Moves a [ROWS x 128] bf16 tile with THREADS threads (THREADS / 64 wavefronts): wavefront w
 // moves the 4 tile rows of every 1 KB region n * WAVES + w.
 template <int ROWS, int THREADS>

@@ -18,7 +18,7 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpith_hip.so")
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 
-SOURCES = ["api.hip", "combine.hip", "attn_fwd.hip", "attn_fwd_d128.hip", "attn_bwd_dq.hip", "attn_bwd_dkdv.hip"]
+SOURCES = ["api.hip", "combine.hip", "attn_fwd.hip", "attn_fwd_d128.hip", "attn_bwd_dq.hip", "attn_bwd_dkdv.hip", "attn_bwd_dkdv_d128.hip"]
 
 # -packed-fp32-ops is switched off on purpose: some packed fp32 forms have produced wrong results
 # on the target machines. Code object v5 is understood by both the ROCm 7.0 runtime bundled with
@@ -58,7 +58,7 @@ def _compile(src: str, extra: list) -> str:
 def build(verbose: bool = True, extra_flags=()) -> str:
     """Compiles every HIP source and links libpith_hip.so. Returns the library path."""
     os.makedirs(OBJ_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
     # libamdhip64 is referenced by soname only (no rpath): inside a PyTorch process the loader
     # then resolves it to the HIP runtime PyTorch has already loaded instead of a second copy.

@@ -165,6 +165,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   auto matrix_block = [&](const char* stage_prev, const char* stage_cur) __attribute__((always_inline)) {
     constexpr int NT = 4 * DB, NS = 2 * KS;
     static_assert(kAhead <= NT, "look-ahead assumes it starts inside the gradient product");
+    __builtin_amdgcn_s_setprio(2);  // the wave that owns the matrix pipe issues first
     bf16x8 at[4][DB], as[KS][2];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -203,6 +204,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(0);
   };
 
   // A: x = S of query tile mt -> P, left in the exchange buffer (fp32) and in frag (bf16).
@@ -242,19 +245,22 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
                                       x[rb][8 * jj + 4], x[rb][8 * jj + 5], x[rb][8 * jj + 6], x[rb][8 * jj + 7]);
     }
   };
-  // B: x = dP of the tile in `stage`, P from the exchange buffer -> dS in frag (bf16)
+  // B: x = dP of the tile in `stage`, P from the exchange buffer -> dS / scale in frag (bf16).
+  // The factor `scale` of dS is applied once to the accumulated dK in the epilogue.
   auto make_ds = [&](const char* stage) __attribute__((always_inline)) {
     const float* delta_s = reinterpret_cast<const float*>(stage + 2 * kTile) + kBM;
+    f32x4 pr[2][4], d4[2][4];
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
-      f32x4 pr[4], d4[4];
+    for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int b4 = 0; b4 < 4; ++b4) {
-        pr[b4] = *reinterpret_cast<const f32x4*>(exch + ((rb * 4 + b4) * 64 + lane) * 16);
-        d4[b4] = *reinterpret_cast<const f32x4*>(delta_s + 32 * rb + 8 * b4 + 4 * g);
+        pr[rb][b4] = *reinterpret_cast<const f32x4*>(exch + ((rb * 4 + b4) * 64 + lane) * 16);
+        d4[rb][b4] = *reinterpret_cast<const f32x4*>(delta_s + 32 * rb + 8 * b4 + 4 * g);
       }
 #pragma unroll
-      for (int v = 0; v < 16; ++v) x[rb][v] = pr[v >> 2][v & 3] * (x[rb][v] - d4[v >> 2][v & 3]) * p.scale;
+    for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x[rb][v] = pr[rb][v >> 2][v & 3] * (x[rb][v] - d4[rb][v >> 2][v & 3]);
 #pragma unroll
       for (int jj = 0; jj < 2; ++jj)
         frag[2 * rb + jj] = to_bf16x8(x[rb][8 * jj], x[rb][8 * jj + 1], x[rb][8 * jj + 2], x[rb][8 * jj + 3],
@@ -265,55 +271,75 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far: tile 0, stationary fragments
   __syncthreads();
 
-  // Interval i = 0 .. n_iter touches tiles i-1 and i; tile -1 and tile n_iter do not exist.
+  // Interval i = 0 .. n_iter touches tiles i-1 and i; tile -1 and tile n_iter do not exist, so the
+  // first and the last interval are peeled and the loop body in between is straight-line code.
+  // Under the causal mask a tile that lies entirely above a pair's diagonal is processed like any
+  // other: its P is all zeros (at most one tile per query head and pair).
   // Ring stages rotate: prev <- cur <- next <- (the stage prev used to be).
   auto run = [&](auto role_tag) __attribute__((always_inline)) {
     constexpr bool ROLE_B = decltype(role_tag)::value;
     TileCursor cur = {hq0, m_first};
-    bool prev_active = false;
     int off_prev = 2 * kStage, off_cur = 0, off_next = kStage;
-    for (int i = 0; i <= n_iter; ++i) {
-      const char* stage_cur = smem + off_cur;
-      const char* stage_prev = smem + off_prev;
-      const bool have_cur = i < n_iter;
-      // under the causal mask a pair skips the tiles that lie entirely above its diagonal
-      const bool cur_active = have_cur && (!CAUSAL || cur.mt * kBM + kBM > kv_pair0);
-      const bool will_request = i + 1 < n_iter;
-      if (!ROLE_B) {
-        if (prev_active && cur_active) matrix_block(stage_prev, stage_cur);
-        else {
-          if (prev_active) transposed_product(stage_prev);
-          if (cur_active) straight_product(stage_cur);
-        }
-        __syncthreads();  // B has read P(i-1); the matrix pipe passes to B
-        if (will_request) request(smem + off_next);
-        if (cur_active) make_p(stage_cur, cur.mt);
-      } else {
-        if (will_request) request(smem + off_next);
-        if (prev_active) make_ds(stage_prev);
-        __syncthreads();
-        if (prev_active && cur_active) matrix_block(stage_prev, stage_cur);
-        else {
-          if (prev_active) transposed_product(stage_prev);
-          if (cur_active) straight_product(stage_cur);
-        }
-      }
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // tile i+1 has landed
+    auto end_interval = [&]() __attribute__((always_inline)) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // the tile requested in this interval has landed
       __syncthreads();
-      prev_active = cur_active;
-      if (have_cur) cur.advance(m_first, m_end);
+      cur.advance(m_first, m_end);
       const int t = off_prev;
       off_prev = off_cur;
       off_cur = off_next;
       off_next = t;
+    };
+    // interval 0
+    if (!ROLE_B) {
+      straight_product(smem + off_cur);
+      __syncthreads();
+      if (n_iter > 1) request(smem + off_next);
+      make_p(smem + off_cur, cur.mt);
+    } else {
+      if (n_iter > 1) request(smem + off_next);
+      __syncthreads();
+      straight_product(smem + off_cur);
+    }
+    end_interval();
+    for (int i = 1; i < n_iter; ++i) {
+      const char* stage_cur = smem + off_cur;
+      const char* stage_prev = smem + off_prev;
+      const bool will_request = i + 1 < n_iter;
+      if (!ROLE_B) {
+        matrix_block(stage_prev, stage_cur);
+        __syncthreads();  // B has read P(i-1); the matrix pipe passes to B
+        if (will_request) request(smem + off_next);
+        make_p(stage_cur, cur.mt);
+      } else {
+        if (will_request) request(smem + off_next);
+        make_ds(stage_prev);
+        __syncthreads();
+        matrix_block(stage_prev, stage_cur);
+      }
+      end_interval();
+    }
+    // interval n_iter
+    if (!ROLE_B) {
+      transposed_product(smem + off_prev);
+      __syncthreads();
+    } else {
+      make_ds(smem + off_prev);
+      __syncthreads();
+      transposed_product(smem + off_prev);
     }
   };
-  // Both roles pass the same barriers; separate loops keep each body straight-line.
+  // Both roles pass the same barriers; separate code keeps each loop body straight-line.
   if (n_iter > 0) {
     if (!role_b) run(std::false_type{});
     else run(std::true_type{});
   }
 
+  if (role_b) {
+#pragma unroll
+    for (int o = 0; o < DB; ++o)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[o][v] *= p.scale;
+  }
   // ---- epilogue: wave A stores dV, wave B stores dK, for key row `key`, features 32*o + 8*b4 + 4*g ..+3
   if (key < p.Skv) {
     if (p.split > 1) {

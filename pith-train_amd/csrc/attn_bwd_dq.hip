@@ -190,12 +190,17 @@ void launch_dq(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
   p.accumulate = a->accumulate_dq;
   const dim3 grid((unsigned)(p.tiles * a->Hq * a->B)), block(WAVES * 64);
   const bool f32 = a->dq_dtype == PITH_F32;
-  if (a->causal) {
-    if (f32) hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV, true, QB, NB, WAVES, float>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV, true, QB, NB, WAVES, __bf16>), grid, block, 0, st, p);
+  if constexpr (DQK == 128 && DV == 128) {
+    static_assert(BM == 256, "the 128-dim kernel owns 256 query rows per workgroup");
+    launch_dq_d128(p, a->causal != 0, f32, st);
   } else {
-    if (f32) hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV, false, QB, NB, WAVES, float>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV, false, QB, NB, WAVES, __bf16>), grid, block, 0, st, p);
+    if (a->causal) {
+      if (f32) hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV, true, QB, NB, WAVES, float>), grid, block, 0, st, p);
+      else hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV, true, QB, NB, WAVES, __bf16>), grid, block, 0, st, p);
+    } else {
+      if (f32) hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV, false, QB, NB, WAVES, float>), grid, block, 0, st, p);
+      else hipLaunchKernelGGL((attn_bwd_dq_kernel<DQK, DV, false, QB, NB, WAVES, __bf16>), grid, block, 0, st, p);
+    }
   }
 }
 

@@ -126,126 +126,144 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
   };
   // ---- dQ^T += K^T dS^T of one tile
   auto accumulate = [&](const char* ktile) __attribute__((always_inline)) {
+    bf16x8 at[4][DB];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int o = 0; o < DB; ++o) {
         const char* base = ktile + j * 16 * kRowBytes128;
-        const bf16x8 a = lds_read_transposed_at(base + t_off[o][0], base + t_off[o][1]);
-        acc[o] = mfma32(a, dsf[j], acc[o]);
-      }
-  };
-  // ---- both, as one block with the fragment reads kAhead products ahead
-  auto matrix_block = [&](const char* kprev, const char* ktile, const char* vtile) __attribute__((always_inline)) {
-    constexpr int NT = 4 * DB, NS = 4 * KS;
-    static_assert(kAhead <= NT, "look-ahead assumes it starts inside the gradient product");
-    bf16x8 at[4][DB], ak[KS][2], av[KS][2];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int o = 0; o < DB; ++o) {
-        const char* base = kprev + j * 16 * kRowBytes128;
         at[j][o] = lds_read_transposed_at(base + t_off[o][0], base + t_off[o][1]);
       }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) ak[ks][nb] = *reinterpret_cast<const bf16x8*>(ktile + s_off[ks] + nb * 32 * kRowBytes128);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) av[ks][nb] = *reinterpret_cast<const bf16x8*>(vtile + s_off[ks] + nb * 32 * kRowBytes128);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int o = 0; o < DB; ++o) acc[o] = mfma32(at[j][o], dsf[j], acc[o]);
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        s[nb][v] = 0.f;
-        dp[nb][v] = 0.f;
-      }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) s[nb] = mfma32(ak[ks][nb], qf[ks], s[nb]);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) dp[nb] = mfma32(av[ks][nb], dof[ks], dp[nb]);
-    // a transposed fragment takes two LDS reads, a straight one a single read
     __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
 #pragma unroll
-    for (int m = 0; m < NT - kAhead; ++m) {
+    for (int m = 0; m < 4 * DB - kAhead; ++m) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
-#pragma unroll
-    for (int m = 0; m < NS; ++m) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
     __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
   };
-  // ---- S, dP of tile t -> dS / scale as bf16 fragments
-  auto make_ds = [&](int t) __attribute__((always_inline)) {
+  // ---- half nb (32 keys) of tile t: s[nb], dp[nb] -> dS / scale as bf16 fragments dsf[2*nb], dsf[2*nb+1]
+  auto make_ds_half_masked = [&](int t, int nb) __attribute__((always_inline)) {
     const int n0 = t * kBN;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) s[nb][v] = __builtin_amdgcn_exp2f(s[nb][v] * p.kappa - lse_q);
+    for (int v = 0; v < 16; ++v) s[nb][v] = __builtin_amdgcn_exp2f(s[nb][v] * p.kappa - lse_q);
     if ((CAUSAL && (n0 + kBN - 1 > q_wave0)) || (n0 + kBN > p.Skv)) {
       // tile crossing the diagonal of a causal chunk, or a ragged last tile (wave-uniform branch)
       const int limit = CAUSAL ? min(qrow, p.Skv - 1) : p.Skv - 1;  // last visible key
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v)
-          if (n0 + nb * 32 + acc_row(v, g) > limit) s[nb][v] = 0.f;
+      for (int v = 0; v < 16; ++v)
+        if (n0 + nb * 32 + acc_row(v, g) > limit) s[nb][v] = 0.f;
     }
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int v = 0; v < 16; ++v) s[nb][v] *= dp[nb][v] - delta_q;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s[nb][v] *= dp[nb][v] - delta_q;
+    for (int jj = 0; jj < 2; ++jj)
+      dsf[2 * nb + jj] = to_bf16x8(s[nb][8 * jj], s[nb][8 * jj + 1], s[nb][8 * jj + 2], s[nb][8 * jj + 3],
+                                   s[nb][8 * jj + 4], s[nb][8 * jj + 5], s[nb][8 * jj + 6], s[nb][8 * jj + 7]);
+  };
+  // ---- S^T and dP^T of one half (32 keys) of a tile, with the dS arithmetic of the unmasked
+  // half `other` of a tile already scored (-1: none) woven in: after every pair of MFMAs come the
+  // exp / multiply / convert of two elements, so that the matrix pipe keeps running while this
+  // wave converts scores. The order is pinned with scheduling barriers; the LDS fragment reads
+  // run kAhead / 2 contraction steps ahead.
+  auto scores_half = [&](const char* ktile, const char* vtile, int nb, int other) __attribute__((always_inline)) {
+    constexpr int kPre = kAhead / 2;
+    bf16x8 ak[KS], av[KS];
+    uint32_t w[8];
 #pragma unroll
-      for (int jj = 0; jj < 2; ++jj)
-        dsf[2 * nb + jj] = to_bf16x8(s[nb][8 * jj], s[nb][8 * jj + 1], s[nb][8 * jj + 2], s[nb][8 * jj + 3],
-                                     s[nb][8 * jj + 4], s[nb][8 * jj + 5], s[nb][8 * jj + 6], s[nb][8 * jj + 7]);
+    for (int ks = 0; ks < kPre; ++ks) {
+      ak[ks] = *reinterpret_cast<const bf16x8*>(ktile + s_off[ks] + nb * 32 * kRowBytes128);
+      av[ks] = *reinterpret_cast<const bf16x8*>(vtile + s_off[ks] + nb * 32 * kRowBytes128);
     }
+    f32x16 sn, dn;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      sn[v] = 0.f;
+      dn[v] = 0.f;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + kPre < KS) {
+        ak[ks + kPre] = *reinterpret_cast<const bf16x8*>(ktile + s_off[ks + kPre] + nb * 32 * kRowBytes128);
+        av[ks + kPre] = *reinterpret_cast<const bf16x8*>(vtile + s_off[ks + kPre] + nb * 32 * kRowBytes128);
+      }
+      sn = mfma32(ak[ks], qf[ks], sn);
+      dn = mfma32(av[ks], dof[ks], dn);
+      // empty volatile statements pin the program order: the optimiser would otherwise sink the
+      // arithmetic below past all MFMAs
+      asm volatile("" : "+v"(sn), "+v"(dn));
+      if (other >= 0) {
+        const float e0 = __builtin_amdgcn_exp2f(s[other][2 * ks] * p.kappa - lse_q) * (dp[other][2 * ks] - delta_q);
+        const float e1 = __builtin_amdgcn_exp2f(s[other][2 * ks + 1] * p.kappa - lse_q) * (dp[other][2 * ks + 1] - delta_q);
+        w[ks] = pack_bf16x2(e0, e1);
+        asm volatile("" : "+v"(w[ks]));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (other >= 0) {
+      const u32x4 lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};
+      dsf[2 * other] = __builtin_bit_cast(bf16x8, lo);
+      dsf[2 * other + 1] = __builtin_bit_cast(bf16x8, hi);
+    }
+    s[nb] = sn;
+    dp[nb] = dn;
   };
 
   __builtin_amdgcn_s_waitcnt(0x0F70);  // tile 0 and the stationary fragments
   __syncthreads();
 
   // Interval i = 0 .. n_tiles_wg touches tiles i-1 and i. A wave has work up to interval
-  // n_tiles_wave; every wave passes all barriers.
+  // n_tiles_wave; every wave passes all barriers. Between intervals a wave carries S, dP of the
+  // upper half (keys 32..63) of the last tile and the dS fragments of its lower half: the vector
+  // arithmetic of a half tile is issued between the MFMAs that produce the next half, so that
+  // the matrix pipe does not idle while a wave converts scores.
   auto end_interval = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // the tiles requested in this interval have landed
     __syncthreads();
   };
+  auto kslot = [&](int t) __attribute__((always_inline)) { return kbuf + (t & (kKSlots - 1)) * kTile; };
+  auto vslot = [&](int t) __attribute__((always_inline)) { return vbuf + (t & (kVSlots - 1)) * kTile; };
+  // tiles [0, first_masked) need no mask for this wave
+  int first_masked = p.Skv / kBN;
+  if (CAUSAL) first_masked = min(first_masked, q_wave0 >= kBN - 1 ? (q_wave0 - (kBN - 1)) / kBN + 1 : 0);
+  const int n_fast = min(n_tiles_wave, first_masked);
+
   // interval 0 (every wave has at least one tile)
-  scores(kbuf, vbuf);
+  scores(kslot(0), vslot(0));
   if (1 < n_tiles_wg) request(1);
-  make_ds(0);
+  make_ds_half_masked(0, 0);
   end_interval();
   int i = 1;
-  for (; i < n_tiles_wave; ++i) {
-    matrix_block(kbuf + ((i - 1) & (kKSlots - 1)) * kTile, kbuf + (i & (kKSlots - 1)) * kTile,
-                 vbuf + (i & (kVSlots - 1)) * kTile);
+  for (; i < n_fast; ++i) {  // tiles i-1 and i unmasked
+    scores_half(kslot(i), vslot(i), 0, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    accumulate(kslot(i - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    scores_half(kslot(i), vslot(i), 1, 0);
     __builtin_amdgcn_sched_barrier(0);
     if (i + 1 < n_tiles_wg) request(i + 1);
-    make_ds(i);
+    end_interval();
+  }
+  for (; i < n_tiles_wave; ++i) {  // near the diagonal / ragged end: plain order, masks applied
+    make_ds_half_masked(i - 1, 1);
+    accumulate(kslot(i - 1));
+    scores(kslot(i), vslot(i));
+    if (i + 1 < n_tiles_wg) request(i + 1);
+    make_ds_half_masked(i, 0);
     end_interval();
   }
   // interval n_tiles_wave: the last gradient product of this wave
-  accumulate(kbuf + ((i - 1) & (kKSlots - 1)) * kTile);
-  if (i <= n_tiles_wg - 1) {
-    // other waves of the workgroup still have tiles to visit: keep moving them and keep in step
-    for (; i < n_tiles_wg; ++i) {
-      if (i + 1 < n_tiles_wg) request(i + 1);
-      end_interval();
-    }
+  make_ds_half_masked(i - 1, 1);
+  accumulate(kslot(i - 1));
+  // other waves of the workgroup may still have tiles to visit: keep moving them and keep in step
+  for (; i < n_tiles_wg; ++i) {
+    if (i + 1 < n_tiles_wg) request(i + 1);
+    end_interval();
   }
 
   OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * kD;

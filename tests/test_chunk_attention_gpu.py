@@ -38,6 +38,15 @@ CASES = [  # B, Sq, Skv, Hq, Hkv, Dqk, Dv, causal
     pytest.param(1, 77, 77, 2, 2, 192, 128, True, id="ragged-mla-77-causal"),
     pytest.param(1, 1, 1, 1, 1, 64, 64, True, id="single-token"),
     pytest.param(1, 2048, 2048, 4, 1, 128, 128, True, id="gqa-4/1-s2048-causal"),
+    # edges of the pipelined 128-dim kernels: one / two / three tiles, tile boundaries +- 1
+    pytest.param(1, 1, 1, 1, 1, 128, 128, True, id="d128-single-token"),
+    pytest.param(1, 64, 64, 2, 2, 128, 128, True, id="d128-one-tile-causal"),
+    pytest.param(1, 65, 65, 2, 1, 128, 128, True, id="d128-65-causal"),
+    pytest.param(1, 129, 64, 2, 2, 128, 128, False, id="d128-sq129-skv64"),
+    pytest.param(1, 64, 129, 4, 4, 128, 128, False, id="d128-sq64-skv129"),
+    pytest.param(1, 193, 193, 8, 1, 128, 128, True, id="d128-193-causal-gqa8"),
+    pytest.param(2, 320, 448, 8, 2, 128, 128, False, id="d128-b2-320x448"),
+    pytest.param(1, 640, 640, 2, 2, 128, 128, True, id="d128-640-causal"),
 ]
 
 

@@ -239,7 +239,7 @@ def main():
         "fwd": {"ms": round(ms_fwd, 4), "tflops": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2)},
         "bwd": {"ms": round(ms_bwd, 4), "tflops": round(bwd_flops / (ms_bwd * 1e-3) / 1e12, 2)},
         "roofline": {
-            "kernel": "attn_bwd_dkdv_kernel<128,128,non-causal> (S, dP, dV, dK of one ring step)",
+            "kernel": "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step)",
             "bound": "mfma", "achieved": round(dkdv_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
             "ms_per_launch": round(ms_dkdv, 4),

@@ -35,6 +35,12 @@ HQ, HKV, DQK, DV, S_LOCAL, CP, RANK = 32, 4, 128, 128, 8192, 4, 1
 LAYOUT = "zigzag"
 
 
+# HBM bytes of one launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes
+# (`--counter-pass`), scaled by what the same counters read for a plain copy of known size:
+# profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt (215.6 MB read + 67.1 MB written).
+DKDV_TRAFFIC_BYTES = 282_700_000
+
+
 def make_inputs(torch, device):
     g = torch.Generator().manual_seed(42)
     s = DQK**-0.5
@@ -116,6 +122,16 @@ def bench_ring(torch, args, dev_inputs):
             attn_bwd_dkdv_into(*a, scale, False)
 
     dkdv_launches()
+    if args.counter_pass:
+        # rocprofv3 --pmc run: a few more launches of the roofline kernel and a plain elementwise
+        # copy of known size (256 MiB read, 256 MiB written) to calibrate the counter against
+        dkdv_launches()
+        src = torch.ones(64 << 20, dtype=torch.float32, device=q.device)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        return None
     ms_dkdv = time_events(torch, dkdv_launches, args.steps) / len(launches)
     entries = (S_LOCAL * S_LOCAL // 2) * HQ
     dkdv_flops = 2 * (2 * DQK + 2 * DV) * entries
@@ -181,6 +197,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--counter-pass", action="store_true",
+                    help="run only the roofline kernel and a calibration copy (for rocprofv3 --pmc), print no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit(
@@ -195,7 +213,11 @@ def main():
     torch.cuda.set_device(device)
 
     host_inputs, dev_inputs = make_inputs(torch, device)
-    ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops = bench_ring(torch, args, dev_inputs)
+    ring = bench_ring(torch, args, dev_inputs)
+    if ring is None:
+        print("counter pass done")
+        return
+    ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops = ring
     fwd_flops, bwd_flops = flops_per_step()
     tflops = (fwd_flops + bwd_flops) / (ms_step * 1e-3) / 1e12
     ms_comb, comb_bytes, comb_host = bench_combine(torch, device)
@@ -241,7 +263,7 @@ def main():
         "roofline": {
             "kernel": "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step)",
             "bound": "mfma", "achieved": round(dkdv_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+            "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": DKDV_TRAFFIC_BYTES,
             "ms_per_launch": round(ms_dkdv, 4),
         },  # fmt: skip
         "combine": {

@@ -240,20 +240,22 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
   end_interval();
   int i = 1;
   for (; i < n_fast; ++i) {  // tiles i-1 and i unmasked
+    // tile i+1 is requested first: its slots were last read in interval i-1, and the load then
+    // has the whole interval to land
+    if (i + 1 < n_tiles_wg) request(i + 1);
     scores_half(kslot(i), vslot(i), 0, 1);
     __builtin_amdgcn_sched_barrier(0);
     accumulate(kslot(i - 1));
     __builtin_amdgcn_sched_barrier(0);
     scores_half(kslot(i), vslot(i), 1, 0);
     __builtin_amdgcn_sched_barrier(0);
-    if (i + 1 < n_tiles_wg) request(i + 1);
     end_interval();
   }
   for (; i < n_tiles_wave; ++i) {  // near the diagonal / ragged end: plain order, masks applied
+    if (i + 1 < n_tiles_wg) request(i + 1);
     make_ds_half_masked(i - 1, 1);
     accumulate(kslot(i - 1));
     scores(kslot(i), vslot(i));
-    if (i + 1 < n_tiles_wg) request(i + 1);
     make_ds_half_masked(i, 0);
     end_interval();
   }

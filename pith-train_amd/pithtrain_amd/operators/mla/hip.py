@@ -177,25 +177,67 @@ def _mla_bwd_dq(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, dout: torch.T
     return dq_out
 
 
-class _CausalAttentionFunc(torch.autograd.Function):
-    """Single-device causal attention with the HIP kernels (what MLA.forward differentiates)."""
+# ---------------------------------------------------------------------------------------------
+# Single-device attention as torch.library custom ops, so that layers compiled with
+# torch.compile(fullgraph=True) keep working: the reference wraps its Triton launches the same
+# way (pithtrain/operators/mla/triton.py:445-508). Two ops (forward, backward), fake
+# implementations that only produce shapes, and an autograd formula tying them together.
 
-    @staticmethod
-    def forward(ctx, q, k, v, softmax_scale):
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        o, lse = _mla_fwd(q, k, v, softmax_scale, causal=True)
-        ctx.save_for_backward(q, k, v, o, lse)
-        ctx.softmax_scale = softmax_scale
-        return o
 
-    @staticmethod
-    def backward(ctx, grad_o):
-        q, k, v, o, lse = ctx.saved_tensors
-        grad_o = grad_o.contiguous()
-        delta = _mla_bwd_preprocess(o, grad_o)
-        dk, dv = _mla_bwd_dk_dv(q, k, v, grad_o, lse, delta, ctx.softmax_scale, causal=True)
-        dq = _mla_bwd_dq(q, k, v, grad_o, lse, delta, ctx.softmax_scale, causal=True)
-        return dq, dk, dv, None
+@torch.library.custom_op("pithtrain_amd::attn_fwd", mutates_args=())
+def _attn_fwd_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
+                 causal: bool) -> tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
+    return _mla_fwd(q.contiguous(), k.contiguous(), v.contiguous(), softmax_scale, causal)
+
+
+@_attn_fwd_op.register_fake
+def _(q, k, v, softmax_scale, causal):
+    b, sq, hq, _ = q.shape
+    return q.new_empty((b, sq, hq, v.shape[-1])), q.new_empty((b, hq, sq), dtype=torch.float32)
+
+
+@torch.library.custom_op("pithtrain_amd::attn_bwd", mutates_args=())
+def _attn_bwd_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
+                 dout: torch.Tensor, softmax_scale: float,
+                 causal: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:  # fmt: skip
+    q, k, v, o, dout = q.contiguous(), k.contiguous(), v.contiguous(), o.contiguous(), dout.contiguous()
+    delta = _mla_bwd_preprocess(o, dout)
+    dk, dv = _mla_bwd_dk_dv(q, k, v, dout, lse, delta, softmax_scale, causal)
+    dq = _mla_bwd_dq(q, k, v, dout, lse, delta, softmax_scale, causal)
+    return dq, dk, dv
+
+
+@_attn_bwd_op.register_fake
+def _(q, k, v, o, lse, dout, softmax_scale, causal):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
+def _attn_setup_context(ctx, inputs, output):
+    q, k, v, softmax_scale, causal = inputs
+    o, lse = output
+    ctx.save_for_backward(q, k, v, o, lse)
+    ctx.softmax_scale = softmax_scale
+    ctx.causal = causal
+
+
+def _attn_backward(ctx, grad_o, grad_lse):
+    q, k, v, o, lse = ctx.saved_tensors
+    dq, dk, dv = _attn_bwd_op(q, k, v, o, lse, grad_o, ctx.softmax_scale, ctx.causal)
+    return dq, dk, dv, None, None
+
+
+_attn_fwd_op.register_autograd(_attn_backward, setup_context=_attn_setup_context)
+
+
+def attention_func(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float | None = None,
+                   causal: bool = False) -> torch.Tensor:  # fmt: skip
+    """Attention on one device (no context parallelism) with autograd: the call that replaces
+    flash_attn_func(q, k, v, softmax_scale=..., causal=...) at pithtrain/models/qwen3_30b_a3b.py:424-430.
+    q [b, sq, hq, d], k/v [b, skv, hkv, d] bf16 (hq a multiple of hkv); returns o [b, sq, hq, dv] bf16."""
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** -0.5
+    o, _ = _attn_fwd_op(q, k, v, softmax_scale, causal)
+    return o
 
 
 class MLA(nn.Module):
@@ -222,10 +264,11 @@ class MLA(nn.Module):
         )
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
-        return _CausalAttentionFunc.apply(q, k, v, self.softmax_scale)
+        o, _ = _attn_fwd_op(q, k, v, self.softmax_scale, True)
+        return o
 
 
 __all__ = [
-    "MLA", "_mla_fwd", "_mla_bwd_preprocess", "_mla_bwd_dk_dv", "_mla_bwd_dq",
+    "MLA", "attention_func", "_mla_fwd", "_mla_bwd_preprocess", "_mla_bwd_dk_dv", "_mla_bwd_dq",
     "attn_fwd_into", "attn_bwd_delta_into", "attn_bwd_dkdv_into", "attn_bwd_dq_into",
 ]  # fmt: skip

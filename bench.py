@@ -14,6 +14,8 @@ HBM before the timed region. One JSON line is printed:
   roofline   the dominant kernel (non-causal dK/dV), timed per launch with events on the launch stream
   combine    the log2 combine at [1,4096,32,128] bf16+bf16 -> fp32 over rotating buffers, GB/s of
              algorithmic bytes against the 8 TB/s HBM peak, with its own roofline
+  norm_rope  the layer's prologue (per-head RMSNorm + rotary embedding of q [1,8192,32,128] and
+             k [1,8192,4,128], forward and backward) over rotating buffers, GB/s of algorithmic bytes
   cpu_baseline  the oracle's eager-PyTorch restatement of the same ring share, timed on the host
              cores over one kv-head group (8 of the 32 query heads)
 """
@@ -166,6 +168,66 @@ def bench_combine(torch, device, reps=50):
     return ms, nbytes, host
 
 
+def bench_norm_rope(torch, device, reps=40):
+    """Forward and backward of the q and k prologue at one rank's shape; every buffer is read or
+    written once per launch, so algorithmic bytes = sum of the tensors' sizes."""
+    from pithtrain_amd.operators.norm_rope import norm_rope_bwd_into, norm_rope_fwd_into
+
+    g = torch.Generator().manual_seed(7)
+    bf = torch.bfloat16
+    cos = torch.randn(1, S_LOCAL, DQK, generator=g).to(bf).to(device)
+    sin = torch.randn(1, S_LOCAL, DQK, generator=g).to(bf).to(device)
+    sets = []
+    for _ in range(5):  # 5 x 302 MB of q-sized tensors > the 256 MiB last-level cache
+        per_tensor = []
+        for h in (HQ, HKV):
+            x = torch.randn(1, S_LOCAL, h, DQK, generator=g).to(bf).to(device)
+            dout = torch.randn(1, S_LOCAL, h, DQK, generator=g).to(bf).to(device)
+            w = (torch.rand(DQK, generator=g) + 0.5).to(bf).to(device)
+            per_tensor.append((x, w, dout, torch.empty_like(x), torch.empty_like(x),
+                               torch.empty(DQK, dtype=torch.float32, device=device)))  # fmt: skip
+        sets.append(per_tensor)
+    size = lambda *ts: sum(t.numel() * t.element_size() for t in ts)  # noqa: E731
+    fwd_bytes = sum(size(x, w, out, cos, sin) for x, w, _, out, _, _ in sets[0])
+    bwd_bytes = sum(size(x, w, dout, dx, dw, cos, sin) for x, w, dout, _, dx, dw in sets[0])
+    it = [0]
+
+    def forward():
+        for x, w, _, out, _, _ in sets[it[0] % len(sets)]:
+            norm_rope_fwd_into(x, w, cos, sin, out, 1e-6)
+        it[0] += 1
+
+    def backward():
+        for x, w, dout, _, dx, dw in sets[it[0] % len(sets)]:
+            norm_rope_bwd_into(x, w, cos, sin, dout, dx, dw, 1e-6)
+        it[0] += 1
+
+    for _ in range(5):
+        forward()
+        backward()
+    ms_f = time_events(torch, forward, reps)
+    ms_b = time_events(torch, backward, reps)
+    host = [t.cpu() for t in sets[0][0][:3]] + [cos.cpu(), sin.cpu()]
+    return ms_f, fwd_bytes, ms_b, bwd_bytes, host
+
+
+def cpu_baseline_norm_rope(torch, host, reps=3):
+    """The oracle's fp32 forward + backward of the q tensor on the host cores; GB/s of the same
+    algorithmic byte count."""
+    from oracle import prologue_oracle as P
+
+    x, w, dout, cos, sin = host
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        P.norm_rope_fwd(x, w, cos, sin, 1e-6, dtype=torch.float32)
+        P.norm_rope_bwd(x, w, cos, sin, dout, 1e-6, dtype=torch.float32)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    nbytes = 5 * x.numel() * 2 + 4 * cos.numel() * 2  # x, out | x, dout, dx; cos and sin twice
+    return nbytes / times[len(times) // 2] / 1e9
+
+
 def cpu_baseline_ring(torch, host_inputs):
     from oracle import ring_oracle as R
 
@@ -222,10 +284,13 @@ def main():
     tflops = (fwd_flops + bwd_flops) / (ms_step * 1e-3) / 1e12
     ms_comb, comb_bytes, comb_host = bench_combine(torch, device)
     comb_gbps = comb_bytes / (ms_comb * 1e-3) / 1e9
+    nr_ms_f, nr_bytes_f, nr_ms_b, nr_bytes_b, nr_host = bench_norm_rope(torch, device)
+    nr_gbps = (nr_bytes_f + nr_bytes_b) / ((nr_ms_f + nr_ms_b) * 1e-3) / 1e9
 
     cores = torch.get_num_threads()
     cpu = None
     combine_cpu = None
+    norm_rope_cpu = None
     if not args.no_cpu_baseline:
         cpu_tflops, cpu_s = cpu_baseline_ring(torch, host_inputs)
         cpu = {
@@ -236,6 +301,10 @@ def main():
         combine_cpu = {
             "value": round(cpu_baseline_combine(torch, comb_host, comb_bytes), 2), "unit": "GB/s", "cores": cores,
             "kind": "port", "sample": "full [1,4096,32,128] combine, eager PyTorch, median of 5",
+        }  # fmt: skip
+        norm_rope_cpu = {
+            "value": round(cpu_baseline_norm_rope(torch, nr_host), 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "q tensor [1,8192,32,128] only, forward + backward, fp32 eager PyTorch, median of 3",
         }  # fmt: skip
 
     dkdv_tflops = dkdv_flops / (ms_dkdv * 1e-3) / 1e12
@@ -273,6 +342,17 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": round(comb_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
             "cpu_baseline": combine_cpu,
+        },  # fmt: skip
+        "norm_rope": {
+            "metric": "q/k RMSNorm + rotary embedding fwd+bwd GB/s (q [1,8192,32,128] + k [1,8192,4,128] bf16)",
+            "value": round(nr_gbps, 1), "unit": "GB/s",
+            "fwd": {"us": round(nr_ms_f * 1e3, 2), "bytes": nr_bytes_f,
+                    "gbps": round(nr_bytes_f / (nr_ms_f * 1e-3) / 1e9, 1)},
+            "bwd": {"us": round(nr_ms_b * 1e3, 2), "bytes": nr_bytes_b,
+                    "gbps": round(nr_bytes_b / (nr_ms_b * 1e-3) / 1e9, 1)},
+            "roofline": {"bound": "hbm", "achieved": round(nr_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(nr_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+            "cpu_baseline": norm_rope_cpu,
         },  # fmt: skip
         "cpu_baseline": cpu,
     }

@@ -22,6 +22,7 @@
  *   pithtrain/operators/ring_attention/standard.py:91-93,134-153   flash-attn _flash_attn_forward / _flash_attn_backward call sites
  *   pithtrain/operators/ring_attention/mla.py:27-40  _online_softmax_combine_log2
  *   pithtrain/operators/ring_attention/standard.py:53-66  _online_softmax_combine
+ *   pithtrain/models/qwen3_30b_a3b.py:417-421        q_norm / k_norm + apply_rotary_pos_emb (the step before the path)
  */
 #ifndef PITH_HIP_H
 #define PITH_HIP_H
@@ -172,6 +173,41 @@ int64_t pith_attn_bwd_dkdv_workspace_bytes(const pith_attn_bwd_args* args);
  * `.to(q.dtype)` on an fp32 accumulator (ring_attention/mla.py:78, standard.py:104) when the
  * last combine did not already emit bf16. n must be a multiple of 8. */
 int pith_cast_f32_bf16(const float* src, void* dst, int64_t n, pith_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Attention prologue of the GQA layer: per-head RMSNorm followed by the rotary embedding,
+ *     y   = x * rsqrt(mean_d(x^2) + eps) * weight          (each [b, s, h] row of D elements)
+ *     out = y * cos + rotate_half(y) * sin,  rotate_half(y) = cat(-y[D/2:], y[:D/2])
+ * Replaces q_norm / k_norm (torch.nn.RMSNorm over the head dim) and apply_rotary_pos_emb at
+ * pithtrain/models/qwen3_30b_a3b.py:417-421 (definitions :100-136, :381-382); called once for q
+ * and once for k. weight == NULL skips the normalisation (apply_rotary_pos_emb alone).
+ * x, out, dout [B,S,H,D] bf16; cos, sin [B,S,D] bf16 with batch stride cs_bs (0 = one [S,D]
+ * table shared by all batch elements); weight [D] bf16 or fp32. Arithmetic is fp32 with one
+ * rounding to bf16 at the end. D must be 8 * a power of two, at most 512; pointers and batch
+ * strides must keep 8-byte alignment. `out` may alias x (forward) or dout (backward).
+ * Backward: `out` receives dx; with a weight, dweight [D] fp32 is overwritten with the sum over
+ * all rows, added in a fixed order through `workspace` (size from
+ * pith_norm_rope_bwd_workspace_bytes; required then). The forward ignores dout, dweight and the
+ * workspace. */
+typedef struct {
+  const void* x;
+  const void* weight;
+  const void* cos;
+  const void* sin;
+  const void* dout;
+  void* out;
+  float* dweight;
+  void* workspace;
+  int64_t workspace_bytes;
+  int64_t B, S, H, D;
+  int64_t x_bs, out_bs, dout_bs, cs_bs; /* batch strides, elements */
+  float eps;
+  int32_t weight_dtype; /* PITH_BF16 | PITH_F32 */
+} pith_norm_rope_args;
+
+int pith_norm_rope_fwd(const pith_norm_rope_args* args, pith_stream_t stream);
+int pith_norm_rope_bwd(const pith_norm_rope_args* args, pith_stream_t stream);
+int64_t pith_norm_rope_bwd_workspace_bytes(const pith_norm_rope_args* args);
 
 #ifdef __cplusplus
 }

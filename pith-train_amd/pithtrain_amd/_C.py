@@ -81,6 +81,16 @@ class AttnBwdArgs(Structure):
     ]  # fmt: skip
 
 
+class NormRopeArgs(Structure):
+    _fields_ = [
+        ("x", c_void_p), ("weight", c_void_p), ("cos", c_void_p), ("sin", c_void_p), ("dout", c_void_p),
+        ("out", c_void_p), ("dweight", c_void_p), ("workspace", c_void_p), ("workspace_bytes", c_int64),
+        ("B", c_int64), ("S", c_int64), ("H", c_int64), ("D", c_int64),
+        ("x_bs", c_int64), ("out_bs", c_int64), ("dout_bs", c_int64), ("cs_bs", c_int64),
+        ("eps", c_float), ("weight_dtype", c_int32),
+    ]  # fmt: skip
+
+
 # name -> (restype, argtypes); must list every symbol declared in include/pith_hip.h
 SYMBOLS = {
     "pith_version": (c_int, []),
@@ -93,6 +103,9 @@ SYMBOLS = {
     "pith_attn_bwd_dq": (c_int, [POINTER(AttnBwdArgs), c_void_p]),
     "pith_attn_bwd_dkdv_workspace_bytes": (c_int64, [POINTER(AttnBwdArgs)]),
     "pith_cast_f32_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "pith_norm_rope_fwd": (c_int, [POINTER(NormRopeArgs), c_void_p]),
+    "pith_norm_rope_bwd": (c_int, [POINTER(NormRopeArgs), c_void_p]),
+    "pith_norm_rope_bwd_workspace_bytes": (c_int64, [POINTER(NormRopeArgs)]),
 }
 
 _lib = None
@@ -164,6 +177,6 @@ def bhs_strides(t: torch.Tensor, what: str):
 
 
 __all__ = [
-    "lib", "check", "PithError", "CombineArgs", "AttnFwdArgs", "AttnDeltaArgs", "AttnBwdArgs", "SYMBOLS",
+    "lib", "check", "PithError", "CombineArgs", "AttnFwdArgs", "AttnDeltaArgs", "AttnBwdArgs", "NormRopeArgs", "SYMBOLS",
     "dtype_code", "current_stream", "require_device", "bshd_batch_stride", "bhs_strides", "byref",
 ]  # fmt: skip

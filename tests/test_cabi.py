@@ -40,6 +40,7 @@ def test_struct_layouts_match_the_header(tmp_path):
         "pith_attn_fwd_args": _C.AttnFwdArgs,
         "pith_attn_delta_args": _C.AttnDeltaArgs,
         "pith_attn_bwd_args": _C.AttnBwdArgs,
+        "pith_norm_rope_args": _C.NormRopeArgs,
     }
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "pith_hip.h"', "int main(void){"]
     for cname, st in pairs.items():
@@ -118,6 +119,54 @@ def test_combine_and_bwd_validation():
     assert lib.pith_attn_bwd_delta(ctypes.byref(d), None) == _C.PITH_ERR_UNSUPPORTED
 
 
+def _norm_rope_args(**kw):
+    base = dict(x=16, weight=16, cos=16, sin=16, dout=16, out=16, dweight=16, workspace=None, workspace_bytes=0,
+                B=2, S=64, H=4, D=128, x_bs=64 * 4 * 128, out_bs=64 * 4 * 128, dout_bs=64 * 4 * 128, cs_bs=64 * 128,
+                eps=1e-6, weight_dtype=_C.PITH_BF16)  # fmt: skip
+    base.update(kw)
+    return _C.NormRopeArgs(**base)
+
+
+@pytest.mark.parametrize(
+    "kw,code",
+    [
+        (dict(x=None), _C.PITH_ERR_NULL_POINTER),
+        (dict(cos=None), _C.PITH_ERR_NULL_POINTER),
+        (dict(H=0), _C.PITH_ERR_BAD_SHAPE),
+        (dict(D=96), _C.PITH_ERR_UNSUPPORTED),
+        (dict(D=1024), _C.PITH_ERR_UNSUPPORTED),
+        (dict(weight_dtype=9), _C.PITH_ERR_BAD_DTYPE),
+        (dict(x=12), _C.PITH_ERR_MISALIGNED),
+        (dict(cs_bs=6), _C.PITH_ERR_MISALIGNED),
+        (dict(x_bs=1024), _C.PITH_ERR_BAD_SHAPE),
+        (dict(cs_bs=128), _C.PITH_ERR_BAD_SHAPE),
+    ],
+)
+def test_norm_rope_rejects_bad_arguments(kw, code):
+    lib = _C.lib()
+    for fn in (lib.pith_norm_rope_fwd, lib.pith_norm_rope_bwd):
+        rc = fn(ctypes.byref(_norm_rope_args(**kw)), None)
+        assert rc == code, lib.pith_last_error()
+        assert lib.pith_last_error().startswith(b"pith_norm_rope")
+
+
+def test_norm_rope_backward_needs_its_workspace():
+    lib = _C.lib()
+    assert lib.pith_norm_rope_fwd(None, None) == _C.PITH_ERR_NULL_POINTER
+    assert lib.pith_norm_rope_bwd(None, None) == _C.PITH_ERR_NULL_POINTER
+    a = _norm_rope_args()
+    need = lib.pith_norm_rope_bwd_workspace_bytes(ctypes.byref(a))
+    assert need > 0 and need % (128 * 4) == 0
+    assert lib.pith_norm_rope_bwd(ctypes.byref(a), None) == _C.PITH_ERR_BAD_SHAPE  # no workspace given
+    assert b"workspace" in lib.pith_last_error()
+    a.workspace, a.workspace_bytes = 16, need - 4
+    assert lib.pith_norm_rope_bwd(ctypes.byref(a), None) == _C.PITH_ERR_BAD_SHAPE
+    assert lib.pith_norm_rope_bwd(ctypes.byref(_norm_rope_args(dout=None)), None) == _C.PITH_ERR_NULL_POINTER
+    assert lib.pith_norm_rope_bwd(ctypes.byref(_norm_rope_args(dweight=None)), None) == _C.PITH_ERR_NULL_POINTER
+    # without a weight there is nothing to reduce, hence no workspace
+    assert lib.pith_norm_rope_bwd_workspace_bytes(ctypes.byref(_norm_rope_args(weight=None))) == 0
+
+
 def test_operators_refuse_cpu_tensors():
     """No CPU fallback: the product path raises instead of computing somewhere else."""
     import torch
@@ -131,6 +180,12 @@ def test_operators_refuse_cpu_tensors():
     lse = torch.zeros(1, 2, 64)
     with pytest.raises(RuntimeError, match="need tensors on a GPU"):
         _online_softmax_combine_log2(q, lse, q, lse)
+    from pithtrain_amd.operators.norm_rope import qk_norm_rope
+
+    w = torch.ones(128, dtype=torch.bfloat16)
+    cs = torch.zeros(1, 64, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="need tensors on a GPU"):
+        qk_norm_rope(q, q, w, w, cs, cs, 1e-6)
 
 
 def test_ring_schedule_matches_oracle_schedule():

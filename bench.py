@@ -171,7 +171,7 @@ def bench_combine(torch, device, reps=50):
 def bench_norm_rope(torch, device, reps=40):
     """Forward and backward of the q and k prologue at one rank's shape; every buffer is read or
     written once per launch, so algorithmic bytes = sum of the tensors' sizes."""
-    from pithtrain_amd.operators.norm_rope import norm_rope_bwd_into, norm_rope_fwd_into
+    from pithtrain_amd.operators.norm_rope import qk_norm_rope_bwd_into, qk_norm_rope_fwd_into
 
     g = torch.Generator().manual_seed(7)
     bf = torch.bfloat16
@@ -192,14 +192,14 @@ def bench_norm_rope(torch, device, reps=40):
     bwd_bytes = sum(size(x, w, dout, dx, dw, cos, sin) for x, w, dout, _, dx, dw in sets[0])
     it = [0]
 
-    def forward():
-        for x, w, _, out, _, _ in sets[it[0] % len(sets)]:
-            norm_rope_fwd_into(x, w, cos, sin, out, 1e-6)
+    def forward():  # q and k in one launch
+        (q, wq, _, q_out, _, _), (k, wk, _, k_out, _, _) = sets[it[0] % len(sets)]
+        qk_norm_rope_fwd_into(q, k, wq, wk, cos, sin, q_out, k_out, 1e-6)
         it[0] += 1
 
-    def backward():
-        for x, w, dout, _, dx, dw in sets[it[0] % len(sets)]:
-            norm_rope_bwd_into(x, w, cos, sin, dout, dx, dw, 1e-6)
+    def backward():  # one launch plus the fixed-order sum of the dweight partials
+        (q, wq, gq, _, dq, dwq), (k, wk, gk, _, dk, dwk) = sets[it[0] % len(sets)]
+        qk_norm_rope_bwd_into(q, k, wq, wk, cos, sin, gq, gk, dq, dk, dwq, dwk, 1e-6)
         it[0] += 1
 
     for _ in range(5):

@@ -209,6 +209,13 @@ int pith_norm_rope_fwd(const pith_norm_rope_args* args, pith_stream_t stream);
 int pith_norm_rope_bwd(const pith_norm_rope_args* args, pith_stream_t stream);
 int64_t pith_norm_rope_bwd_workspace_bytes(const pith_norm_rope_args* args);
 
+/* The same for two tensors in ONE launch each way: q and k of a layer, which the reference
+ * handles together (pithtrain/models/qwen3_30b_a3b.py:417-421). Results are identical to two
+ * single-tensor calls. The two argument structs are independent (own H, weight, workspace, even
+ * cos/sin) except that B must agree and either both or neither has a weight. */
+int pith_norm_rope_fwd_pair(const pith_norm_rope_args* a, const pith_norm_rope_args* b, pith_stream_t stream);
+int pith_norm_rope_bwd_pair(const pith_norm_rope_args* a, const pith_norm_rope_args* b, pith_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,7 +23,8 @@ namespace pith {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kBatch = 4;  // rows a slot has in flight
+constexpr int kBatch = 4;  // rows a slot has in flight (forward)
+constexpr int kBwdBatch = 2;  // the same in the backward, which holds two tensors per row
 
 struct Quad {  // four consecutive bf16
   u32x2 raw;
@@ -52,9 +53,18 @@ struct NormRopeParams {
   int lanes;   // D / 8, a power of two <= 64
   int hg;      // head groups per token, a power of two <= 2048 / D
   int tile_s;  // tokens per block = (2048 / D) / hg
+  int n_tiles;  // ceil(S / tile_s)
+  int grid_x;  // blocks of this tensor along x (backward: blocks stride over the tiles)
   int64_t x_bs, out_bs, dout_bs, cs_bs;
   float eps, inv_d;
   int w_f32;
+};
+
+// One launch serves up to two tensors (q and k of a layer): blocks [0, blocks0) along x work on
+// t[0], the rest on t[1].
+struct PairParams {
+  NormRopeParams t[2];
+  int blocks0;
 };
 
 __device__ __forceinline__ float row_sum(float v, int lanes) {
@@ -84,12 +94,15 @@ __device__ __forceinline__ void load_gain(const NormRopeParams& p, int l, float*
 }
 
 template <bool NORM>
-__global__ __launch_bounds__(kThreads) void norm_rope_fwd_kernel(NormRopeParams p) {
+__global__ __launch_bounds__(kThreads) void norm_rope_fwd_kernel(PairParams pp) {
+  const int which = (int)blockIdx.x >= pp.blocks0;
+  const NormRopeParams& p = pp.t[which];
+  const int bx = blockIdx.x - (which ? pp.blocks0 : 0);
   const int l = threadIdx.x % p.lanes;
   const int slot = threadIdx.x / p.lanes;
   const int g = slot % p.hg;
   const int b = blockIdx.y;
-  const int64_t s = (int64_t)blockIdx.x * p.tile_s + slot / p.hg;
+  const int64_t s = (int64_t)bx * p.tile_s + slot / p.hg;
   if (s >= p.S) return;  // no block-wide synchronisation below
   const int half = p.D >> 1;
 
@@ -161,8 +174,11 @@ __global__ __launch_bounds__(kThreads) void norm_rope_fwd_kernel(NormRopeParams 
 // its rows, the block adds its slots through LDS and writes one [D] partial; a second kernel adds
 // the partials in a fixed order, so dw does not depend on scheduling.
 template <bool NORM>
-__global__ __launch_bounds__(kThreads) void norm_rope_bwd_kernel(NormRopeParams p, int n_tiles) {
+__global__ __launch_bounds__(kThreads) void norm_rope_bwd_kernel(PairParams pp) {
   __shared__ float red[2048];  // [slots][D] = 256 threads x 8 sums
+  const int which = (int)blockIdx.x >= pp.blocks0;
+  const NormRopeParams& p = pp.t[which];
+  const int bx = blockIdx.x - (which ? pp.blocks0 : 0);
   const int l = threadIdx.x % p.lanes;
   const int slot = threadIdx.x / p.lanes;
   const int g = slot % p.hg;
@@ -173,7 +189,7 @@ __global__ __launch_bounds__(kThreads) void norm_rope_bwd_kernel(NormRopeParams 
   float dw_lo[4] = {0.f, 0.f, 0.f, 0.f}, dw_hi[4] = {0.f, 0.f, 0.f, 0.f};
   if (NORM) load_gain(p, l, w_lo, w_hi);
 
-  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+  for (int tile = bx; tile < p.n_tiles; tile += p.grid_x) {
     const int64_t s = (int64_t)tile * p.tile_s + slot / p.hg;
     if (s >= p.S) continue;
     const int64_t cs = b * p.cs_bs + s * p.D + 4 * l;
@@ -188,10 +204,10 @@ __global__ __launch_bounds__(kThreads) void norm_rope_bwd_kernel(NormRopeParams 
     const __bf16* dout = p.dout + b * p.dout_bs + row0;
     __bf16* dx = p.out + b * p.out_bs + row0;
 
-    for (int h0 = g; h0 < p.H; h0 += kBatch * p.hg) {
-      Quad lo[kBatch], hi[kBatch], g_lo[kBatch], g_hi[kBatch];
+    for (int h0 = g; h0 < p.H; h0 += kBwdBatch * p.hg) {
+      Quad lo[kBwdBatch], hi[kBwdBatch], g_lo[kBwdBatch], g_hi[kBwdBatch];
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
+      for (int u = 0; u < kBwdBatch; ++u) {
         const int h = h0 + u * p.hg;
         if (h < p.H) {
           if (NORM) {
@@ -203,7 +219,7 @@ __global__ __launch_bounds__(kThreads) void norm_rope_bwd_kernel(NormRopeParams 
         }
       }
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
+      for (int u = 0; u < kBwdBatch; ++u) {
         const int h = h0 + u * p.hg;
         if (h >= p.H) break;
         float dy_lo[4], dy_hi[4];
@@ -259,7 +275,7 @@ __global__ __launch_bounds__(kThreads) void norm_rope_bwd_kernel(NormRopeParams 
     }
     __syncthreads();
     const int slots = kThreads / p.lanes;
-    float* part = p.partial + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * p.D;
+    float* part = p.partial + ((int64_t)blockIdx.y * p.grid_x + bx) * p.D;
     for (int d = threadIdx.x; d < p.D; d += kThreads) {
       float acc = 0.f;
       for (int sl = 0; sl < slots; ++sl) acc += red[sl * p.D + d];
@@ -273,16 +289,24 @@ __global__ __launch_bounds__(kThreads) void norm_rope_bwd_kernel(NormRopeParams 
 // of additions is fixed, so the result does not depend on scheduling.
 constexpr int kSumCols = 16;
 
-__global__ __launch_bounds__(kThreads) void sum_partials_kernel(const float* __restrict__ partial, float* __restrict__ dw,
-                                                               int n, int D) {
+struct SumParams {
+  const float* partial[2];
+  float* dw[2];
+  int n[2];
+  int D[2];
+};
+
+__global__ __launch_bounds__(kThreads) void sum_partials_kernel(SumParams sp) {
   __shared__ float red[kThreads];
   constexpr int kParts = kThreads / kSumCols;
+  const int t = blockIdx.y;  // tensor of the pair
+  const int n = sp.n[t], D = sp.D[t];
   const int c = threadIdx.x % kSumCols;
   const int col = blockIdx.x * kSumCols + c;
   const int part = threadIdx.x / kSumCols;
   float acc = 0.f;
   if (col < D) {
-    const float* src = partial + col;
+    const float* src = sp.partial[t] + col;
     int i = part;
     for (; i + 7 * kParts < n; i += 8 * kParts) {
       float v[8];
@@ -298,7 +322,7 @@ __global__ __launch_bounds__(kThreads) void sum_partials_kernel(const float* __r
   if (part == 0 && col < D) {
     float total = 0.f;
     for (int i = 0; i < kParts; ++i) total += red[i * kSumCols + c];
-    dw[col] = total;
+    sp.dw[t][col] = total;
   }
 }
 
@@ -363,7 +387,7 @@ NormRopeParams make_params(const pith_norm_rope_args* a, const Plan& pl) {
   p.x = (const __bf16*)a->x; p.w = a->weight; p.cos = (const __bf16*)a->cos; p.sin = (const __bf16*)a->sin;
   p.dout = (const __bf16*)a->dout; p.out = (__bf16*)a->out; p.partial = nullptr;
   p.S = a->S; p.H = (int)a->H; p.D = (int)a->D;
-  p.lanes = pl.lanes; p.hg = pl.hg; p.tile_s = pl.tile_s;
+  p.lanes = pl.lanes; p.hg = pl.hg; p.tile_s = pl.tile_s; p.n_tiles = pl.n_tiles; p.grid_x = pl.n_tiles;
   p.x_bs = a->x_bs; p.out_bs = a->out_bs; p.dout_bs = a->dout_bs; p.cs_bs = a->cs_bs;
   p.eps = a->eps; p.inv_d = 1.0f / (float)a->D;
   p.w_f32 = a->weight_dtype == PITH_F32;
@@ -375,16 +399,104 @@ NormRopeParams make_params(const pith_norm_rope_args* a, const Plan& pl) {
 
 using namespace pith;
 
-extern "C" int pith_norm_rope_fwd(const pith_norm_rope_args* a, pith_stream_t stream) {
-  if (const int rc = validate("pith_norm_rope_fwd", a, false)) return rc;
-  const Plan pl = make_plan(a->B, a->S, a->H, a->D);
-  const NormRopeParams p = make_params(a, pl);
-  const dim3 grid((unsigned)pl.n_tiles, (unsigned)a->B);
+namespace {
+
+// What the two tensors of a pair must agree on: the grid's batch dimension and the kernel variant.
+int validate_pair(const char* who, const pith_norm_rope_args* a, const pith_norm_rope_args* b) {
+  if (a->B != b->B) return fail(PITH_ERR_BAD_SHAPE, "%s: the two tensors differ in B (%lld, %lld)", who, (long long)a->B, (long long)b->B);
+  if ((a->weight == nullptr) != (b->weight == nullptr))
+    return fail(PITH_ERR_UNSUPPORTED, "%s: either both tensors have a weight or neither", who);
+  return PITH_OK;
+}
+
+// `b` may be NULL (one tensor).
+int launch_fwd(const char* who, const pith_norm_rope_args* a, const pith_norm_rope_args* b, pith_stream_t stream) {
+  if (const int rc = validate(who, a, false)) return rc;
+  if (b) {
+    if (const int rc = validate(who, b, false)) return rc;
+    if (const int rc = validate_pair(who, a, b)) return rc;
+  }
+  PairParams pp;
+  const Plan pa = make_plan(a->B, a->S, a->H, a->D);
+  pp.t[0] = make_params(a, pa);
+  pp.t[1] = pp.t[0];
+  pp.blocks0 = pa.n_tiles;
+  int64_t blocks = pa.n_tiles;
+  if (b) {
+    const Plan pb = make_plan(b->B, b->S, b->H, b->D);
+    pp.t[1] = make_params(b, pb);
+    blocks += pb.n_tiles;
+  }
+  const dim3 grid((unsigned)blocks, (unsigned)a->B);
   if (a->weight)
-    hipLaunchKernelGGL(norm_rope_fwd_kernel<true>, grid, dim3(kThreads), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(norm_rope_fwd_kernel<true>, grid, dim3(kThreads), 0, (hipStream_t)stream, pp);
   else
-    hipLaunchKernelGGL(norm_rope_fwd_kernel<false>, grid, dim3(kThreads), 0, (hipStream_t)stream, p);
-  return check_launch("pith_norm_rope_fwd");
+    hipLaunchKernelGGL(norm_rope_fwd_kernel<false>, grid, dim3(kThreads), 0, (hipStream_t)stream, pp);
+  return check_launch(who);
+}
+
+int prepare_bwd(const char* who, const pith_norm_rope_args* a, NormRopeParams* p) {
+  const Plan pl = make_plan(a->B, a->S, a->H, a->D);
+  *p = make_params(a, pl);
+  p->grid_x = bwd_blocks_x(pl, a->B);
+  if (!a->weight) return PITH_OK;
+  const int64_t need = (int64_t)p->grid_x * a->B * a->D * (int64_t)sizeof(float);
+  if (!a->workspace || a->workspace_bytes < need)
+    return fail(PITH_ERR_BAD_SHAPE, "%s: workspace of %lld bytes needed, %lld given", who, (long long)need,
+                (long long)(a->workspace ? a->workspace_bytes : 0));
+  if (reinterpret_cast<uintptr_t>(a->workspace) % 4 || reinterpret_cast<uintptr_t>(a->dweight) % 4)
+    return fail(PITH_ERR_MISALIGNED, "%s: workspace / dweight must be 4-byte aligned", who);
+  p->partial = (float*)a->workspace;
+  return PITH_OK;
+}
+
+int launch_bwd(const char* who, const pith_norm_rope_args* a, const pith_norm_rope_args* b, pith_stream_t stream) {
+  if (const int rc = validate(who, a, true)) return rc;
+  if (b) {
+    if (const int rc = validate(who, b, true)) return rc;
+    if (const int rc = validate_pair(who, a, b)) return rc;
+  }
+  PairParams pp;
+  if (const int rc = prepare_bwd(who, a, &pp.t[0])) return rc;
+  pp.t[1] = pp.t[0];
+  pp.blocks0 = pp.t[0].grid_x;
+  int64_t blocks = pp.blocks0;
+  if (b) {
+    if (const int rc = prepare_bwd(who, b, &pp.t[1])) return rc;
+    blocks += pp.t[1].grid_x;
+  }
+  const dim3 grid((unsigned)blocks, (unsigned)a->B);
+  hipStream_t st = (hipStream_t)stream;
+  if (!a->weight) {
+    hipLaunchKernelGGL(norm_rope_bwd_kernel<false>, grid, dim3(kThreads), 0, st, pp);
+    return check_launch(who);
+  }
+  hipLaunchKernelGGL(norm_rope_bwd_kernel<true>, grid, dim3(kThreads), 0, st, pp);
+  if (const int rc = check_launch(who)) return rc;
+  SumParams sp;
+  const pith_norm_rope_args* both[2] = {a, b ? b : a};
+  int64_t max_d = 0;
+  for (int t = 0; t < 2; ++t) {
+    sp.partial[t] = pp.t[t].partial;
+    sp.dw[t] = both[t]->dweight;
+    sp.n[t] = (int)(pp.t[t].grid_x * both[t]->B);
+    sp.D[t] = (int)both[t]->D;
+    if (both[t]->D > max_d) max_d = both[t]->D;
+  }
+  hipLaunchKernelGGL(sum_partials_kernel, dim3((unsigned)((max_d + kSumCols - 1) / kSumCols), b ? 2u : 1u),
+                     dim3(kThreads), 0, st, sp);
+  return check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int pith_norm_rope_fwd(const pith_norm_rope_args* a, pith_stream_t stream) {
+  return launch_fwd("pith_norm_rope_fwd", a, nullptr, stream);
+}
+
+extern "C" int pith_norm_rope_fwd_pair(const pith_norm_rope_args* a, const pith_norm_rope_args* b, pith_stream_t stream) {
+  if (!a || !b) return fail(PITH_ERR_NULL_POINTER, "pith_norm_rope_fwd_pair: args is NULL");
+  return launch_fwd("pith_norm_rope_fwd_pair", a, b, stream);
 }
 
 extern "C" int64_t pith_norm_rope_bwd_workspace_bytes(const pith_norm_rope_args* a) {
@@ -394,26 +506,10 @@ extern "C" int64_t pith_norm_rope_bwd_workspace_bytes(const pith_norm_rope_args*
 }
 
 extern "C" int pith_norm_rope_bwd(const pith_norm_rope_args* a, pith_stream_t stream) {
-  if (const int rc = validate("pith_norm_rope_bwd", a, true)) return rc;
-  const Plan pl = make_plan(a->B, a->S, a->H, a->D);
-  NormRopeParams p = make_params(a, pl);
-  const int gx = bwd_blocks_x(pl, a->B);
-  const dim3 grid((unsigned)gx, (unsigned)a->B);
-  hipStream_t st = (hipStream_t)stream;
-  if (!a->weight) {
-    hipLaunchKernelGGL(norm_rope_bwd_kernel<false>, grid, dim3(kThreads), 0, st, p, pl.n_tiles);
-    return check_launch("pith_norm_rope_bwd");
-  }
-  const int64_t need = (int64_t)gx * a->B * a->D * (int64_t)sizeof(float);
-  if (!a->workspace || a->workspace_bytes < need)
-    return fail(PITH_ERR_BAD_SHAPE, "pith_norm_rope_bwd: workspace of %lld bytes needed, %lld given", (long long)need,
-                (long long)(a->workspace ? a->workspace_bytes : 0));
-  if (reinterpret_cast<uintptr_t>(a->workspace) % 4 || reinterpret_cast<uintptr_t>(a->dweight) % 4)
-    return fail(PITH_ERR_MISALIGNED, "pith_norm_rope_bwd: workspace / dweight must be 4-byte aligned");
-  p.partial = (float*)a->workspace;
-  hipLaunchKernelGGL(norm_rope_bwd_kernel<true>, grid, dim3(kThreads), 0, st, p, pl.n_tiles);
-  if (const int rc = check_launch("pith_norm_rope_bwd")) return rc;
-  hipLaunchKernelGGL(sum_partials_kernel, dim3((unsigned)((a->D + kSumCols - 1) / kSumCols)), dim3(kThreads), 0, st, p.partial,
-                     a->dweight, (int)(gx * a->B), (int)a->D);
-  return check_launch("pith_norm_rope_bwd (partial sums)");
+  return launch_bwd("pith_norm_rope_bwd", a, nullptr, stream);
+}
+
+extern "C" int pith_norm_rope_bwd_pair(const pith_norm_rope_args* a, const pith_norm_rope_args* b, pith_stream_t stream) {
+  if (!a || !b) return fail(PITH_ERR_NULL_POINTER, "pith_norm_rope_bwd_pair: args is NULL");
+  return launch_bwd("pith_norm_rope_bwd_pair", a, b, stream);
 }

@@ -106,6 +106,8 @@ SYMBOLS = {
     "pith_norm_rope_fwd": (c_int, [POINTER(NormRopeArgs), c_void_p]),
     "pith_norm_rope_bwd": (c_int, [POINTER(NormRopeArgs), c_void_p]),
     "pith_norm_rope_bwd_workspace_bytes": (c_int64, [POINTER(NormRopeArgs)]),
+    "pith_norm_rope_fwd_pair": (c_int, [POINTER(NormRopeArgs), POINTER(NormRopeArgs), c_void_p]),
+    "pith_norm_rope_bwd_pair": (c_int, [POINTER(NormRopeArgs), POINTER(NormRopeArgs), c_void_p]),
 }
 
 _lib = None

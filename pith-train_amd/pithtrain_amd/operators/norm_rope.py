@@ -1,6 +1,7 @@
 """
 Attention prologue of the GQA layer backed by libpith_hip.so: per-head RMSNorm of the projected
-q / k followed by the rotary position embedding, one HIP kernel per tensor and direction.
+q / k followed by the rotary position embedding, one HIP kernel per direction
+(q and k share a launch).
 
 Replaces, at pithtrain/models/qwen3_30b_a3b.py:417-421,
 
@@ -138,16 +139,116 @@ def norm_rope(x: torch.Tensor, weight: Optional[torch.Tensor], cos: torch.Tensor
     return _norm_rope_fwd_op(x, weight, cos, sin, eps)
 
 
+# ---------------------------------------------------------------------------------------------
+# q and k of a layer together: one launch forward, one (plus the dweight sums) backward.
+
+
+def _workspace_for(args: _C.NormRopeArgs, device) -> Optional[torch.Tensor]:
+    need = _C.lib().pith_norm_rope_bwd_workspace_bytes(_C.byref(args))
+    if need == 0:
+        return None
+    workspace = torch.empty(need, dtype=torch.uint8, device=device)
+    args.workspace, args.workspace_bytes = workspace.data_ptr(), need
+    return workspace
+
+
+def qk_norm_rope_fwd_into(q, k, q_weight, k_weight, cos, sin, q_out, k_out, eps: float) -> None:
+    """q_out, k_out <- rope(rms_norm(q) * q_weight), rope(rms_norm(k) * k_weight); weights may both be None."""
+    a = _args(q, q_weight, cos, sin, q_out, eps)
+    b = _args(k, k_weight, cos, sin, k_out, eps)
+    _C.check(_C.lib().pith_norm_rope_fwd_pair(_C.byref(a), _C.byref(b), _C.current_stream(q)))
+
+
+def qk_norm_rope_bwd_into(q, k, q_weight, k_weight, cos, sin, dq_out, dk_out, dq, dk, dq_weight, dk_weight,
+                          eps: float) -> None:  # fmt: skip
+    """dq, dk <- gradients w.r.t. q, k; dq_weight, dk_weight [d] fp32 <- gradients w.r.t. the weights."""
+    a = _args(q, q_weight, cos, sin, dq, eps)
+    b = _args(k, k_weight, cos, sin, dk, eps)
+    keep = []
+    for args, x, w, dout, dweight in ((a, q, q_weight, dq_out, dq_weight), (b, k, k_weight, dk_out, dk_weight)):
+        _C.require_device(x, dout)
+        assert dout.dtype == torch.bfloat16 and dout.shape == x.shape, "a gradient does not match its tensor"
+        args.dout, args.dout_bs = dout.data_ptr(), _C.bshd_batch_stride(dout, "dout")
+        if w is not None:
+            assert dweight is not None and dweight.dtype == torch.float32 and dweight.shape == w.shape, (
+                "dweight must be a float32 tensor shaped like weight"
+            )
+            _C.require_device(x, dweight)
+            assert dweight.is_contiguous(), "dweight is not contiguous"
+            args.dweight = dweight.data_ptr()
+            keep.append(_workspace_for(args, x.device))
+    _C.check(_C.lib().pith_norm_rope_bwd_pair(_C.byref(a), _C.byref(b), _C.current_stream(q)))
+
+
+@torch.library.custom_op("pithtrain_amd::qk_norm_rope_fwd", mutates_args=())
+def _qk_norm_rope_fwd_op(q: torch.Tensor, k: torch.Tensor, q_weight: Optional[torch.Tensor],
+                         k_weight: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor,
+                         eps: float) -> Tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
+    q, k = q.contiguous(), k.contiguous()
+    q_out, k_out = torch.empty_like(q), torch.empty_like(k)
+    qk_norm_rope_fwd_into(q, k, q_weight, k_weight, cos.contiguous(), sin.contiguous(), q_out, k_out, eps)
+    return q_out, k_out
+
+
+@_qk_norm_rope_fwd_op.register_fake
+def _(q, k, q_weight, k_weight, cos, sin, eps):
+    fmt = torch.contiguous_format
+    return torch.empty_like(q, memory_format=fmt), torch.empty_like(k, memory_format=fmt)
+
+
+@torch.library.custom_op("pithtrain_amd::qk_norm_rope_bwd", mutates_args=())
+def _qk_norm_rope_bwd_op(q: torch.Tensor, k: torch.Tensor, q_weight: Optional[torch.Tensor],
+                         k_weight: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor,
+                         dq_out: torch.Tensor, dk_out: torch.Tensor,
+                         eps: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:  # fmt: skip
+    q, k, dq_out, dk_out = q.contiguous(), k.contiguous(), dq_out.contiguous(), dk_out.contiguous()
+    dq, dk = torch.empty_like(q), torch.empty_like(k)
+    # without weights the last two results are empty placeholders (custom ops cannot return None)
+    n = q.shape[-1] if q_weight is not None else 0
+    dwq, dwk = q.new_empty((n,), dtype=torch.float32), q.new_empty((n,), dtype=torch.float32)
+    qk_norm_rope_bwd_into(q, k, q_weight, k_weight, cos.contiguous(), sin.contiguous(), dq_out, dk_out, dq, dk,
+                          dwq if n else None, dwk if n else None, eps)  # fmt: skip
+    return dq, dk, dwq, dwk
+
+
+@_qk_norm_rope_bwd_op.register_fake
+def _(q, k, q_weight, k_weight, cos, sin, dq_out, dk_out, eps):
+    fmt = torch.contiguous_format
+    n = q.shape[-1] if q_weight is not None else 0
+    return (torch.empty_like(q, memory_format=fmt), torch.empty_like(k, memory_format=fmt),
+            q.new_empty((n,), dtype=torch.float32), q.new_empty((n,), dtype=torch.float32))  # fmt: skip
+
+
+def _qk_setup_context(ctx, inputs, output):
+    q, k, q_weight, k_weight, cos, sin, eps = inputs
+    ctx.save_for_backward(q, k, q_weight, k_weight, cos, sin)
+    ctx.eps = eps
+
+
+def _qk_backward(ctx, grad_q, grad_k):
+    q, k, q_weight, k_weight, cos, sin = ctx.saved_tensors
+    dq, dk, dwq, dwk = _qk_norm_rope_bwd_op(q, k, q_weight, k_weight, cos, sin, grad_q, grad_k, ctx.eps)
+    if q_weight is None:
+        return dq, dk, None, None, None, None, None
+    return dq, dk, dwq.to(q_weight.dtype), dwk.to(k_weight.dtype), None, None, None
+
+
+_qk_norm_rope_fwd_op.register_autograd(_qk_backward, setup_context=_qk_setup_context)
+
+
 def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor,
                  cos: torch.Tensor, sin: torch.Tensor, eps: float = 1e-6) -> Tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
-    """The three statements at pithtrain/models/qwen3_30b_a3b.py:417-421 as two kernel launches."""
-    return _norm_rope_fwd_op(q, q_weight, cos, sin, eps), _norm_rope_fwd_op(k, k_weight, cos, sin, eps)
+    """The three statements at pithtrain/models/qwen3_30b_a3b.py:417-421 as one kernel launch."""
+    return _qk_norm_rope_fwd_op(q, k, q_weight, k_weight, cos, sin, eps)
 
 
 def apply_rotary_pos_emb(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor,
                          sin: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
     """pithtrain/models/qwen3_30b_a3b.py:107-136 — same name, arguments and results."""
-    return _norm_rope_fwd_op(q, None, cos, sin, 0.0), _norm_rope_fwd_op(k, None, cos, sin, 0.0)
+    return _qk_norm_rope_fwd_op(q, k, None, None, cos, sin, 0.0)
 
 
-__all__ = ["norm_rope", "qk_norm_rope", "apply_rotary_pos_emb", "norm_rope_fwd_into", "norm_rope_bwd_into"]
+__all__ = [
+    "norm_rope", "qk_norm_rope", "apply_rotary_pos_emb", "norm_rope_fwd_into", "norm_rope_bwd_into",
+    "qk_norm_rope_fwd_into", "qk_norm_rope_bwd_into",
+]  # fmt: skip

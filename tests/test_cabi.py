@@ -163,6 +163,16 @@ def test_norm_rope_backward_needs_its_workspace():
     assert lib.pith_norm_rope_bwd(ctypes.byref(a), None) == _C.PITH_ERR_BAD_SHAPE
     assert lib.pith_norm_rope_bwd(ctypes.byref(_norm_rope_args(dout=None)), None) == _C.PITH_ERR_NULL_POINTER
     assert lib.pith_norm_rope_bwd(ctypes.byref(_norm_rope_args(dweight=None)), None) == _C.PITH_ERR_NULL_POINTER
+    # the two-tensor launch: both structs are validated, B must agree, weights both or neither
+    ok = _norm_rope_args(workspace=16, workspace_bytes=need)
+    assert lib.pith_norm_rope_fwd_pair(ctypes.byref(ok), None, None) == _C.PITH_ERR_NULL_POINTER
+    assert lib.pith_norm_rope_bwd_pair(None, ctypes.byref(ok), None) == _C.PITH_ERR_NULL_POINTER
+    for fn in (lib.pith_norm_rope_fwd_pair, lib.pith_norm_rope_bwd_pair):
+        assert fn(ctypes.byref(ok), ctypes.byref(_norm_rope_args(D=96)), None) == _C.PITH_ERR_UNSUPPORTED
+        other_b = _norm_rope_args(B=3, workspace=16, workspace_bytes=1 << 30)
+        assert fn(ctypes.byref(ok), ctypes.byref(other_b), None) == _C.PITH_ERR_BAD_SHAPE
+        assert b"differ in B" in lib.pith_last_error()
+        assert fn(ctypes.byref(ok), ctypes.byref(_norm_rope_args(weight=None)), None) == _C.PITH_ERR_UNSUPPORTED
     # without a weight there is nothing to reduce, hence no workspace
     assert lib.pith_norm_rope_bwd_workspace_bytes(ctypes.byref(_norm_rope_args(weight=None))) == 0
 

@@ -176,6 +176,51 @@ def test_autograd_and_reference_named_functions(gpu):
     _check(rk, P.norm_rope_fwd(k, None, cos, sin, 0.0), "rope(k)")
 
 
+@pytest.mark.parametrize("with_weight", [True, False])
+def test_pair_launch_equals_two_single_launches(gpu, with_weight):
+    """q and k in one launch: bit-identical to the single-tensor entry points, including dweight."""
+    from pithtrain_amd.operators.norm_rope import (
+        norm_rope_bwd_into, norm_rope_fwd_into, qk_norm_rope_bwd_into, qk_norm_rope_fwd_into,
+    )  # fmt: skip
+
+    b, s, d = 2, 301, 128
+    q, wq, cos, sin, gq = (t.to(gpu) for t in _inputs(b, s, 32, d, seed=51))
+    k, wk, _, _, gk = (t.to(gpu) for t in _inputs(b, s, 4, d, seed=52, weight_dtype=torch.float32))
+    if not with_weight:
+        wq = wk = None
+    new = lambda t: torch.full_like(t, float("nan"))  # noqa: E731
+    dw = lambda: torch.full((d,), float("nan"), device=gpu) if with_weight else None  # noqa: E731
+    single = {"q": new(q), "k": new(k), "dq": new(q), "dk": new(k), "dwq": dw(), "dwk": dw()}
+    norm_rope_fwd_into(q, wq, cos, sin, single["q"], 1e-6)
+    norm_rope_fwd_into(k, wk, cos, sin, single["k"], 1e-6)
+    norm_rope_bwd_into(q, wq, cos, sin, gq, single["dq"], single["dwq"], 1e-6)
+    norm_rope_bwd_into(k, wk, cos, sin, gk, single["dk"], single["dwk"], 1e-6)
+    pair = {"q": new(q), "k": new(k), "dq": new(q), "dk": new(k), "dwq": dw(), "dwk": dw()}
+    qk_norm_rope_fwd_into(q, k, wq, wk, cos, sin, pair["q"], pair["k"], 1e-6)
+    qk_norm_rope_bwd_into(q, k, wq, wk, cos, sin, gq, gk, pair["dq"], pair["dk"], pair["dwq"], pair["dwk"], 1e-6)
+    for name in single:
+        if single[name] is not None:
+            assert torch.equal(single[name], pair[name]), name
+
+
+def test_pair_with_different_head_dims_and_lengths(gpu):
+    """The two tensors of a pair only share B: different S, H, D and cos/sin tables are allowed."""
+    from pithtrain_amd.operators.norm_rope import norm_rope_fwd_into
+    from pithtrain_amd import _C
+    from pithtrain_amd.operators import norm_rope as NR
+
+    xa, wa, ca, sa, _ = (t.to(gpu) for t in _inputs(1, 50, 6, 64, seed=61))
+    xb, wb, cb, sb, _ = (t.to(gpu) for t in _inputs(1, 9, 3, 256, seed=62))
+    oa, ob = torch.empty_like(xa), torch.empty_like(xb)
+    a = NR._args(xa, wa, ca, sa, oa, 1e-6)
+    b = NR._args(xb, wb, cb, sb, ob, 1e-5)
+    _C.check(_C.lib().pith_norm_rope_fwd_pair(_C.byref(a), _C.byref(b), _C.current_stream(xa)))
+    ra, rb = torch.empty_like(xa), torch.empty_like(xb)
+    norm_rope_fwd_into(xa, wa, ca, sa, ra, 1e-6)
+    norm_rope_fwd_into(xb, wb, cb, sb, rb, 1e-5)
+    assert torch.equal(oa, ra) and torch.equal(ob, rb)
+
+
 def test_at_least_as_accurate_as_the_eager_bf16_expression(gpu):
     """The reference's evaluation (nn.RMSNorm, then the bf16 expression of
     pithtrain/models/qwen3_30b_a3b.py:132-136) run eagerly on the GPU: the fused kernel's error

@@ -16,6 +16,8 @@ HBM before the timed region. One JSON line is printed:
              algorithmic bytes against the 8 TB/s HBM peak, with its own roofline
   norm_rope  the layer's prologue (per-head RMSNorm + rotary embedding of q [1,8192,32,128] and
              k [1,8192,4,128], forward and backward) over rotating buffers, GB/s of algorithmic bytes
+  mla_assemble  the MLA layer's prologue (rotary embedding of the rope parts + assembly of query / key /
+             value states, forward and backward) at [1,4096,16,128+64 | 128], GB/s of algorithmic bytes
   cpu_baseline  the oracle's eager-PyTorch restatement of the same ring share, timed on the host
              cores over one kv-head group (8 of the 32 query heads)
 """
@@ -211,6 +213,51 @@ def bench_norm_rope(torch, device, reps=40):
     return ms_f, fwd_bytes, ms_b, bwd_bytes, host
 
 
+def bench_mla_assemble(torch, device, reps=40):
+    """Forward and backward of the MLA prologue at one rank's share of the 16K configuration."""
+    from pithtrain_amd.operators.mla_assemble import mla_assemble_bwd_into, mla_assemble_fwd_into
+
+    b, s, h, dn, dr, dv, lora = 1, 4096, 16, 128, 64, 128, 512
+    g = torch.Generator().manual_seed(11)
+    bf = torch.bfloat16
+    table = torch.rand(16384, dr // 2, generator=g) * 6.283
+    table = torch.cat((table, table), -1)
+    cos, sin = table.cos().to(bf).to(device), table.sin().to(bf).to(device)
+    pos = (torch.arange(s) + 4096).unsqueeze(0).to(device)
+    sets = []
+    for _ in range(3):  # 3 x 252 MB > the 256 MiB last-level cache
+        q = torch.randn(b, s, h, dn + dr, generator=g).to(bf).to(device)
+        kv = torch.randn(b, s, h, dn + dv, generator=g).to(bf).to(device)
+        a_proj = torch.randn(b, s, lora + dr, generator=g).to(bf).to(device)
+        outs = [torch.empty(b, s, h, d, dtype=bf, device=device) for d in (dn + dr, dn + dr, dv)]
+        grads = [torch.empty(b, s, h, dn + dr, dtype=bf, device=device), torch.empty(b, s, h, dn + dv, dtype=bf, device=device),
+                 torch.empty(b, s, dr, dtype=bf, device=device)]  # fmt: skip
+        sets.append((q, kv, a_proj[..., lora:], outs, grads))
+    size = lambda *ts: sum(t.numel() * t.element_size() for t in ts)  # noqa: E731
+    q, kv, k_pe, outs, grads = sets[0]
+    touched_tables = 2 * s * dr * 2  # the cos and sin rows of this share
+    fwd_bytes = size(q, kv, k_pe, pos, *outs) + touched_tables
+    bwd_bytes = size(pos, *outs, *grads) + touched_tables
+    it = [0]
+
+    def forward():
+        q, kv, k_pe, outs, _ = sets[it[0] % len(sets)]
+        mla_assemble_fwd_into(q, kv, k_pe, cos, sin, pos, *outs)
+        it[0] += 1
+
+    def backward():  # the forward outputs stand in for their gradients (same shapes)
+        _, _, _, outs, grads = sets[it[0] % len(sets)]
+        mla_assemble_bwd_into(*outs, cos, sin, pos, *grads)
+        it[0] += 1
+
+    for _ in range(5):
+        forward()
+        backward()
+    ms_f = time_events(torch, forward, reps)
+    ms_b = time_events(torch, backward, reps)
+    return ms_f, fwd_bytes, ms_b, bwd_bytes
+
+
 def cpu_baseline_norm_rope(torch, host, reps=3):
     """The oracle's fp32 forward + backward of the q tensor on the host cores; GB/s of the same
     algorithmic byte count."""
@@ -286,6 +333,8 @@ def main():
     comb_gbps = comb_bytes / (ms_comb * 1e-3) / 1e9
     nr_ms_f, nr_bytes_f, nr_ms_b, nr_bytes_b, nr_host = bench_norm_rope(torch, device)
     nr_gbps = (nr_bytes_f + nr_bytes_b) / ((nr_ms_f + nr_ms_b) * 1e-3) / 1e9
+    ma_ms_f, ma_bytes_f, ma_ms_b, ma_bytes_b = bench_mla_assemble(torch, device)
+    ma_gbps = (ma_bytes_f + ma_bytes_b) / ((ma_ms_f + ma_ms_b) * 1e-3) / 1e9
 
     cores = torch.get_num_threads()
     cpu = None
@@ -353,6 +402,16 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(nr_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": round(nr_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
             "cpu_baseline": norm_rope_cpu,
+        },  # fmt: skip
+        "mla_assemble": {
+            "metric": "MLA rotary + q/k/v assembly fwd+bwd GB/s ([1,4096,16,192] q, [1,4096,16,256] kv, bf16)",
+            "value": round(ma_gbps, 1), "unit": "GB/s",
+            "fwd": {"us": round(ma_ms_f * 1e3, 2), "bytes": ma_bytes_f,
+                    "gbps": round(ma_bytes_f / (ma_ms_f * 1e-3) / 1e9, 1)},
+            "bwd": {"us": round(ma_ms_b * 1e3, 2), "bytes": ma_bytes_b,
+                    "gbps": round(ma_bytes_b / (ma_ms_b * 1e-3) / 1e9, 1)},
+            "roofline": {"bound": "hbm", "achieved": round(ma_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(ma_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
         },  # fmt: skip
         "cpu_baseline": cpu,
     }

@@ -23,6 +23,7 @@
  *   pithtrain/operators/ring_attention/mla.py:27-40  _online_softmax_combine_log2
  *   pithtrain/operators/ring_attention/standard.py:53-66  _online_softmax_combine
  *   pithtrain/models/qwen3_30b_a3b.py:417-421        q_norm / k_norm + apply_rotary_pos_emb (the step before the path)
+ *   pithtrain/models/deepseek_v2_lite.py:446-454     rotary embedding + q/k assembly of the MLA layer (the same step there)
  */
 #ifndef PITH_HIP_H
 #define PITH_HIP_H
@@ -215,6 +216,45 @@ int64_t pith_norm_rope_bwd_workspace_bytes(const pith_norm_rope_args* args);
  * cos/sin) except that B must agree and either both or neither has a weight. */
 int pith_norm_rope_fwd_pair(const pith_norm_rope_args* a, const pith_norm_rope_args* b, pith_stream_t stream);
 int pith_norm_rope_bwd_pair(const pith_norm_rope_args* a, const pith_norm_rope_args* b, pith_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Attention prologue of the MLA layer: rotary embedding of the rope parts and assembly of the
+ * attention operands. Replaces pithtrain/models/deepseek_v2_lite.py:446-454 and the
+ * value_states.contiguous() of :462/:467 (apply_rotary_pos_emb :173-187, rotate_half :165-169):
+ *     pe'  = de-interleave(pe): pe'[j] = pe[2j], pe'[Dr/2+j] = pe[2j+1]
+ *     rot(pe) = pe' * cos[pos] + rotate_half(pe') * sin[pos]
+ *     q_out = [q[..., :Dn] | rot(q[..., Dn:])]            [B,S,H,Dn+Dr]
+ *     k_out = [kv[..., :Dn] | rot(k_pe) for every head]   [B,S,H,Dn+Dr]
+ *     v_out = kv[..., Dn:]                                [B,S,H,Dv]
+ * q [B,S,H,Dn+Dr] and kv [B,S,H,Dn+Dv] bf16 are contiguous per batch element (batch strides
+ * given); k_pe [B,S,Dr] bf16 has a row stride (it is a column slice of a wider projection);
+ * cos, sin [P,Dr] bf16 tables indexed by position_ids [B,S] int64 (batch stride pos_bs; NULL =
+ * position s). Positions outside [0,P) are clamped. Outputs are contiguous.
+ * Backward: dq_out, dk_out, dv_out are the gradients of the three outputs (contiguous); q_out
+ * receives dq [B,S,H,Dn+Dr], k_out receives dkv [B,S,H,Dn+Dv], v_out receives dk_pe [B,S,Dr]
+ * (summed over heads in head order); q, kv, k_pe are not read.
+ * Dn and Dv must be multiples of 8, Dr of 16; pointers and strides keep 16-byte alignment. */
+typedef struct {
+  const void* q;
+  const void* kv;
+  const void* k_pe;
+  const void* cos;
+  const void* sin;
+  const int64_t* position_ids;
+  void* q_out;
+  void* k_out;
+  void* v_out;
+  const void* dq_out;
+  const void* dk_out;
+  const void* dv_out;
+  int64_t B, S, H, Dn, Dr, Dv, P;
+  int64_t q_bs, kv_bs;        /* batch strides, elements */
+  int64_t k_pe_bs, k_pe_rs;   /* batch and row strides of k_pe, elements */
+  int64_t pos_bs;             /* batch stride of position_ids (0 = shared) */
+} pith_mla_assemble_args;
+
+int pith_mla_assemble_fwd(const pith_mla_assemble_args* args, pith_stream_t stream);
+int pith_mla_assemble_bwd(const pith_mla_assemble_args* args, pith_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -91,6 +91,17 @@ class NormRopeArgs(Structure):
     ]  # fmt: skip
 
 
+class MlaAssembleArgs(Structure):
+    _fields_ = [
+        ("q", c_void_p), ("kv", c_void_p), ("k_pe", c_void_p), ("cos", c_void_p), ("sin", c_void_p),
+        ("position_ids", c_void_p), ("q_out", c_void_p), ("k_out", c_void_p), ("v_out", c_void_p),
+        ("dq_out", c_void_p), ("dk_out", c_void_p), ("dv_out", c_void_p),
+        ("B", c_int64), ("S", c_int64), ("H", c_int64), ("Dn", c_int64), ("Dr", c_int64), ("Dv", c_int64),
+        ("P", c_int64), ("q_bs", c_int64), ("kv_bs", c_int64), ("k_pe_bs", c_int64), ("k_pe_rs", c_int64),
+        ("pos_bs", c_int64),
+    ]  # fmt: skip
+
+
 # name -> (restype, argtypes); must list every symbol declared in include/pith_hip.h
 SYMBOLS = {
     "pith_version": (c_int, []),
@@ -108,6 +119,8 @@ SYMBOLS = {
     "pith_norm_rope_bwd_workspace_bytes": (c_int64, [POINTER(NormRopeArgs)]),
     "pith_norm_rope_fwd_pair": (c_int, [POINTER(NormRopeArgs), POINTER(NormRopeArgs), c_void_p]),
     "pith_norm_rope_bwd_pair": (c_int, [POINTER(NormRopeArgs), POINTER(NormRopeArgs), c_void_p]),
+    "pith_mla_assemble_fwd": (c_int, [POINTER(MlaAssembleArgs), c_void_p]),
+    "pith_mla_assemble_bwd": (c_int, [POINTER(MlaAssembleArgs), c_void_p]),
 }
 
 _lib = None
@@ -179,6 +192,6 @@ def bhs_strides(t: torch.Tensor, what: str):
 
 
 __all__ = [
-    "lib", "check", "PithError", "CombineArgs", "AttnFwdArgs", "AttnDeltaArgs", "AttnBwdArgs", "NormRopeArgs", "SYMBOLS",
+    "lib", "check", "PithError", "CombineArgs", "AttnFwdArgs", "AttnDeltaArgs", "AttnBwdArgs", "NormRopeArgs", "MlaAssembleArgs", "SYMBOLS",
     "dtype_code", "current_stream", "require_device", "bshd_batch_stride", "bhs_strides", "byref",
 ]  # fmt: skip

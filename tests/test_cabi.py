@@ -41,6 +41,7 @@ def test_struct_layouts_match_the_header(tmp_path):
         "pith_attn_delta_args": _C.AttnDeltaArgs,
         "pith_attn_bwd_args": _C.AttnBwdArgs,
         "pith_norm_rope_args": _C.NormRopeArgs,
+        "pith_mla_assemble_args": _C.MlaAssembleArgs,
     }
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "pith_hip.h"', "int main(void){"]
     for cname, st in pairs.items():
@@ -177,6 +178,47 @@ def test_norm_rope_backward_needs_its_workspace():
     assert lib.pith_norm_rope_bwd_workspace_bytes(ctypes.byref(_norm_rope_args(weight=None))) == 0
 
 
+def _mla_assemble_args(**kw):
+    base = dict(q=16, kv=16, k_pe=16, cos=16, sin=16, position_ids=None, q_out=16, k_out=16, v_out=16,
+                dq_out=16, dk_out=16, dv_out=16, B=2, S=8, H=16, Dn=128, Dr=64, Dv=128, P=64,
+                q_bs=8 * 16 * 192, kv_bs=8 * 16 * 256, k_pe_bs=8 * 576, k_pe_rs=576, pos_bs=8)  # fmt: skip
+    base.update(kw)
+    return _C.MlaAssembleArgs(**base)
+
+
+@pytest.mark.parametrize(
+    "kw,code",
+    [
+        (dict(cos=None), _C.PITH_ERR_NULL_POINTER),
+        (dict(q_out=None), _C.PITH_ERR_NULL_POINTER),
+        (dict(S=0), _C.PITH_ERR_BAD_SHAPE),
+        (dict(P=0), _C.PITH_ERR_BAD_SHAPE),
+        (dict(Dr=24), _C.PITH_ERR_UNSUPPORTED),
+        (dict(Dn=100), _C.PITH_ERR_UNSUPPORTED),
+        (dict(sin=8), _C.PITH_ERR_MISALIGNED),
+        (dict(position_ids=4), _C.PITH_ERR_MISALIGNED),
+    ],
+)
+def test_mla_assemble_rejects_bad_arguments(kw, code):
+    lib = _C.lib()
+    for fn in (lib.pith_mla_assemble_fwd, lib.pith_mla_assemble_bwd):
+        rc = fn(ctypes.byref(_mla_assemble_args(**kw)), None)
+        assert rc == code, lib.pith_last_error()
+        assert lib.pith_last_error().startswith(b"pith_mla_assemble")
+
+
+def test_mla_assemble_direction_specific_validation():
+    lib = _C.lib()
+    assert lib.pith_mla_assemble_fwd(None, None) == _C.PITH_ERR_NULL_POINTER
+    assert lib.pith_mla_assemble_bwd(None, None) == _C.PITH_ERR_NULL_POINTER
+    fwd, bwd = lib.pith_mla_assemble_fwd, lib.pith_mla_assemble_bwd
+    assert fwd(ctypes.byref(_mla_assemble_args(kv=None)), None) == _C.PITH_ERR_NULL_POINTER
+    assert bwd(ctypes.byref(_mla_assemble_args(dk_out=None)), None) == _C.PITH_ERR_NULL_POINTER
+    assert fwd(ctypes.byref(_mla_assemble_args(k_pe_rs=32)), None) == _C.PITH_ERR_BAD_SHAPE
+    assert fwd(ctypes.byref(_mla_assemble_args(k_pe_rs=580)), None) == _C.PITH_ERR_MISALIGNED
+    assert fwd(ctypes.byref(_mla_assemble_args(q_bs=1024)), None) == _C.PITH_ERR_BAD_SHAPE
+
+
 def test_operators_refuse_cpu_tensors():
     """No CPU fallback: the product path raises instead of computing somewhere else."""
     import torch
@@ -196,6 +238,13 @@ def test_operators_refuse_cpu_tensors():
     cs = torch.zeros(1, 64, 128, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="need tensors on a GPU"):
         qk_norm_rope(q, q, w, w, cs, cs, 1e-6)
+    from pithtrain_amd.operators.mla_assemble import mla_assemble_qkv
+
+    x = torch.zeros(1, 4, 2, 192, dtype=torch.bfloat16)
+    kv = torch.zeros(1, 4, 2, 256, dtype=torch.bfloat16)
+    table = torch.zeros(8, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="need tensors on a GPU"):
+        mla_assemble_qkv(x, kv, torch.zeros(1, 4, 1, 64, dtype=torch.bfloat16), table, table, None)
 
 
 def test_ring_schedule_matches_oracle_schedule():

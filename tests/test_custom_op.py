@@ -78,3 +78,44 @@ def test_compiled_module_matches_eager(gpu):
     oa.float().square().sum().backward()
     ob.float().square().sum().backward()
     assert torch.equal(qa.grad, qb.grad) and torch.equal(ka.grad, kb.grad) and torch.equal(va.grad, vb.grad)
+
+
+def test_prologue_fake_implementations_and_fullgraph_compile():
+    """The q/k RMSNorm + rotary embedding ops trace without a GPU: a compiled attention layer's
+    prologue + attention chain, shapes and gradients (weights included) on meta tensors."""
+    from pithtrain_amd.operators.norm_rope import apply_rotary_pos_emb, qk_norm_rope
+
+    def layer(q, k, v, wq, wk, cos, sin):
+        q, k = qk_norm_rope(q, k, wq, wk, cos, sin, 1e-6)
+        return attention_func(q, k, v, None, True)
+
+    f = torch.compile(layer, backend="aot_eager", fullgraph=True)
+    q, k, v = _meta(2, 64, 8, 128), _meta(2, 64, 2, 128), _meta(2, 64, 2, 128)
+    wq, wk = _meta(128), _meta(128)
+    cos = torch.empty(2, 64, 128, dtype=torch.bfloat16, device="meta")
+    o = f(q, k, v, wq, wk, cos, cos)
+    assert o.shape == (2, 64, 8, 128)
+    o.sum().backward()
+    assert q.grad.shape == q.shape and k.grad.shape == k.shape
+    assert wq.grad.shape == (128,) and wq.grad.dtype == torch.bfloat16 and wk.grad.shape == (128,)
+    rq, rk = apply_rotary_pos_emb(q.detach(), k.detach(), cos, cos)
+    assert rq.shape == q.shape and rk.shape == k.shape
+
+
+@pytest.mark.gpu
+def test_compiled_prologue_matches_eager(gpu):
+    from pithtrain_amd.operators.norm_rope import qk_norm_rope
+
+    g = torch.Generator().manual_seed(3)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(gpu)  # noqa: E731
+    q, k, wq, wk, cos, sin = mk(1, 200, 32, 128), mk(1, 200, 4, 128), mk(128), mk(128), mk(1, 200, 128), mk(1, 200, 128)
+    f = torch.compile(qk_norm_rope, backend="aot_eager", fullgraph=True)
+    a = [t.clone().requires_grad_() for t in (q, k, wq, wk)]
+    b = [t.clone().requires_grad_() for t in (q, k, wq, wk)]
+    qa, ka = qk_norm_rope(*a, cos, sin, 1e-6)
+    qb, kb = f(*b, cos, sin, 1e-6)
+    assert torch.equal(qa, qb) and torch.equal(ka, kb)
+    (qa.float().square().sum() + ka.float().sum()).backward()
+    (qb.float().square().sum() + kb.float().sum()).backward()
+    for x, y in zip(a, b):
+        assert torch.equal(x.grad, y.grad)

@@ -150,3 +150,89 @@ def test_eager_bf16_composite_is_close_to_the_oracle():
     want = P.norm_rope_fwd(x, norm.weight.detach(), cos, sin, 1e-6)
     err = (eager.double() - want).abs().max().item() / want.abs().max().item()
     assert err < 2e-2
+
+
+# ---------------------------------------------------------------------------------------------
+# MLA layer assembly
+
+
+def _mla_inputs(b, s, h, dn, dr, dv, seed=0, dtype=F64):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b, s, h, dn + dr, generator=g, dtype=dtype)
+    kv = torch.randn(b, s, h, dn + dv, generator=g, dtype=dtype)
+    k_pe = torch.randn(b, s, dr, generator=g, dtype=dtype)
+    theta = torch.rand(64, dr // 2, generator=g, dtype=dtype) * 2 * math.pi  # table of 64 positions
+    pos = torch.randint(0, 64, (b, s), generator=g)
+    return q, kv, k_pe, theta, pos
+
+
+def _independent_mla_forward(q, kv, k_pe, theta, pos, dn):
+    """Index-based de-interleave, rotation in complex arithmetic, slice assignment as in the reference."""
+    b, s, h, _ = q.shape
+    dr = k_pe.shape[-1]
+    phase = torch.polar(torch.ones_like(theta), theta)[pos]  # [B,S,dr/2]
+
+    def rot(pe):  # [..., dr] interleaved pairs
+        z = torch.complex(pe[..., 0::2], pe[..., 1::2]) * (phase if pe.dim() == 3 else phase.unsqueeze(2))
+        return torch.cat((z.real, z.imag), -1)
+
+    query = torch.zeros(b, s, h, dn + dr, dtype=q.dtype)
+    query[..., :dn] = q[..., :dn]
+    query[..., dn:] = rot(q[..., dn:])
+    key = torch.zeros(b, s, h, dn + dr, dtype=q.dtype)
+    key[..., :dn] = kv[..., :dn]
+    key[..., dn:] = rot(k_pe).unsqueeze(2)
+    return query, key, kv[..., dn:]
+
+
+def test_mla_assemble_forward_against_complex_rotation():
+    dn, dr, dv = 16, 8, 24
+    q, kv, k_pe, theta, pos = _mla_inputs(2, 5, 3, dn, dr, dv)
+    full = torch.cat((theta, theta), -1)
+    got = P.mla_assemble_fwd(q, kv, k_pe, full.cos(), full.sin(), pos, dn)
+    want = _independent_mla_forward(q, kv, k_pe, theta, pos, dn)
+    for g_, w_ in zip(got, want):
+        assert torch.allclose(g_, w_, atol=1e-13)
+    assert torch.equal(got[0][..., :dn], q[..., :dn]) and torch.equal(got[2], kv[..., dn:])
+    assert torch.equal(got[1][:, :, 0, dn:], got[1][:, :, 2, dn:])  # the rope part is shared by the heads
+    # positions default to 0..S-1
+    a = P.mla_assemble_fwd(q, kv, k_pe, full.cos(), full.sin(), None, dn)
+    bb = P.mla_assemble_fwd(q, kv, k_pe, full.cos(), full.sin(), torch.arange(5).expand(2, 5), dn)
+    assert all(torch.equal(x, y) for x, y in zip(a, bb))
+
+
+def test_deinterleave_known_values():
+    x = torch.arange(8.0).unsqueeze(0)
+    assert P.deinterleave(x).tolist() == [[0, 2, 4, 6, 1, 3, 5, 7]]
+    assert torch.equal(P._interleave(P.deinterleave(x)), x)
+
+
+def test_mla_assemble_backward_against_autograd_of_an_independent_forward():
+    dn, dr, dv = 8, 8, 16
+    q, kv, k_pe, theta, pos = _mla_inputs(2, 4, 3, dn, dr, dv, seed=4)
+    q.requires_grad_(), kv.requires_grad_(), k_pe.requires_grad_()
+    query, key, value = _independent_mla_forward(q, kv, k_pe, theta, pos, dn)
+    g = torch.Generator().manual_seed(5)
+    dquery, dkey, dvalue = (torch.randn(t.shape, generator=g, dtype=F64) for t in (query, key, value))
+    torch.autograd.backward([query, key, value], [dquery, dkey, dvalue])
+    full = torch.cat((theta, theta), -1)
+    dq, dkv, dk_pe = P.mla_assemble_bwd(dquery, dkey, dvalue, full.cos(), full.sin(), pos, dn)
+    assert torch.allclose(dq, q.grad, atol=1e-12)
+    assert torch.allclose(dkv, kv.grad, atol=1e-12)
+    assert torch.allclose(dk_pe, k_pe.grad, atol=1e-12)
+
+
+def test_mla_assemble_backward_with_tables_that_are_not_rotations():
+    """cos/sin scaled (YaRN mscale) and different in the two halves: autograd through the oracle's
+    own forward, which the previous tests pin, must agree with the closed form."""
+    dn, dr, dv = 8, 16, 8
+    q, kv, k_pe, _, pos = _mla_inputs(1, 6, 2, dn, dr, dv, seed=6)
+    g = torch.Generator().manual_seed(7)
+    cos, sin = torch.randn(64, dr, generator=g, dtype=F64), torch.randn(64, dr, generator=g, dtype=F64)
+    q.requires_grad_(), kv.requires_grad_(), k_pe.requires_grad_()
+    outs = P.mla_assemble_fwd(q, kv, k_pe, cos, sin, pos, dn)
+    grads = [torch.randn(t.shape, generator=g, dtype=F64) for t in outs]
+    torch.autograd.backward(list(outs), grads)
+    dq, dkv, dk_pe = P.mla_assemble_bwd(*grads, cos, sin, pos, dn)
+    assert torch.allclose(dq, q.grad, atol=1e-12) and torch.allclose(dkv, kv.grad, atol=1e-12)
+    assert torch.allclose(dk_pe, k_pe.grad, atol=1e-12)

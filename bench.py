@@ -43,6 +43,10 @@ LAYOUT = "zigzag"
 # (`--counter-pass`), scaled by what the same counters read for a plain copy of known size:
 # profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt (215.6 MB read + 67.1 MB written).
 DKDV_TRAFFIC_BYTES = 282_700_000
+# The same for the HBM-bound kernels: profiles/combine_norm_rope_mla_assemble_hbm_counters.txt
+COMBINE_TRAFFIC_BYTES = 144_900_000
+NORM_ROPE_TRAFFIC_BYTES = 159_400_000 + 235_200_000  # forward + backward launch
+MLA_ASSEMBLE_TRAFFIC_BYTES = 128_000_000 + 128_000_000
 
 
 def make_inputs(torch, device):
@@ -190,8 +194,8 @@ def bench_norm_rope(torch, device, reps=40):
                                torch.empty(DQK, dtype=torch.float32, device=device)))  # fmt: skip
         sets.append(per_tensor)
     size = lambda *ts: sum(t.numel() * t.element_size() for t in ts)  # noqa: E731
-    fwd_bytes = sum(size(x, w, out, cos, sin) for x, w, _, out, _, _ in sets[0])
-    bwd_bytes = sum(size(x, w, dout, dx, dw, cos, sin) for x, w, dout, _, dx, dw in sets[0])
+    fwd_bytes = sum(size(x, w, out) for x, w, _, out, _, _ in sets[0]) + size(cos, sin)
+    bwd_bytes = sum(size(x, w, dout, dx, dw) for x, w, dout, _, dx, dw in sets[0]) + size(cos, sin)
     it = [0]
 
     def forward():  # q and k in one launch
@@ -225,7 +229,7 @@ def bench_mla_assemble(torch, device, reps=40):
     cos, sin = table.cos().to(bf).to(device), table.sin().to(bf).to(device)
     pos = (torch.arange(s) + 4096).unsqueeze(0).to(device)
     sets = []
-    for _ in range(3):  # 3 x 252 MB > the 256 MiB last-level cache
+    for _ in range(5):  # 5 x 127 MB of tensors touched per direction, well beyond the 256 MiB last-level cache
         q = torch.randn(b, s, h, dn + dr, generator=g).to(bf).to(device)
         kv = torch.randn(b, s, h, dn + dv, generator=g).to(bf).to(device)
         a_proj = torch.randn(b, s, lora + dr, generator=g).to(bf).to(device)
@@ -324,6 +328,10 @@ def main():
     host_inputs, dev_inputs = make_inputs(torch, device)
     ring = bench_ring(torch, args, dev_inputs)
     if ring is None:
+        # the HBM-bound kernels, a few dispatches each, for the same counters
+        bench_combine(torch, device, reps=3)
+        bench_norm_rope(torch, device, reps=3)
+        bench_mla_assemble(torch, device, reps=3)
         print("counter pass done")
         return
     ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops = ring
@@ -389,7 +397,7 @@ def main():
             "value": round(comb_gbps, 1), "unit": "GB/s", "us_per_launch": round(ms_comb * 1e3, 2),
             "bytes": comb_bytes,
             "roofline": {"bound": "hbm", "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": round(comb_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+                         "frac": round(comb_gbps / HBM_PEAK_GBPS, 4), "traffic": COMBINE_TRAFFIC_BYTES},
             "cpu_baseline": combine_cpu,
         },  # fmt: skip
         "norm_rope": {
@@ -400,7 +408,7 @@ def main():
             "bwd": {"us": round(nr_ms_b * 1e3, 2), "bytes": nr_bytes_b,
                     "gbps": round(nr_bytes_b / (nr_ms_b * 1e-3) / 1e9, 1)},
             "roofline": {"bound": "hbm", "achieved": round(nr_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": round(nr_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+                         "frac": round(nr_gbps / HBM_PEAK_GBPS, 4), "traffic": NORM_ROPE_TRAFFIC_BYTES},
             "cpu_baseline": norm_rope_cpu,
         },  # fmt: skip
         "mla_assemble": {
@@ -411,7 +419,7 @@ def main():
             "bwd": {"us": round(ma_ms_b * 1e3, 2), "bytes": ma_bytes_b,
                     "gbps": round(ma_bytes_b / (ma_ms_b * 1e-3) / 1e9, 1)},
             "roofline": {"bound": "hbm", "achieved": round(ma_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": round(ma_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+                         "frac": round(ma_gbps / HBM_PEAK_GBPS, 4), "traffic": MLA_ASSEMBLE_TRAFFIC_BYTES},
         },  # fmt: skip
         "cpu_baseline": cpu,
     }

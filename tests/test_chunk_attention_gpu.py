@@ -169,3 +169,43 @@ def test_error_paths(gpu):
     with pytest.raises(AssertionError, match="bfloat16"):
         _mla_fwd(z(1, 64, 2, 128).float(), z(1, 64, 2, 128), z(1, 64, 2, 128), 0.1)
     assert _C.lib().pith_last_error() is not None
+
+
+def _random_cases(n, seed):
+    """Seeded sweep over shapes no hand-picked case covers: odd lengths around and far from tile
+    boundaries, every head-dim family, group sizes 1..8, one or two batch elements."""
+    import random
+
+    rng = random.Random(seed)
+    cases = []
+    for i in range(n):
+        dqk, dv = rng.choice([(128, 128), (128, 128), (192, 128), (64, 64)])
+        causal = rng.random() < 0.5
+        sq = rng.choice([rng.randint(1, 70), rng.randint(60, 270), rng.randint(250, 600)])
+        skv = sq if causal else rng.choice([rng.randint(1, 70), rng.randint(60, 270), rng.randint(250, 600)])
+        hkv = rng.choice([1, 2, 3])
+        group = rng.choice([1, 2, 4, 8])
+        b = rng.choice([1, 1, 2])
+        cases.append(pytest.param(b, sq, skv, hkv * group, hkv, dqk, dv, causal, 1000 + i,
+                                  id=f"rand{i}-b{b}-{sq}x{skv}-h{hkv * group}/{hkv}-d{dqk}-{'c' if causal else 'n'}"))  # fmt: skip
+    return cases
+
+
+@pytest.mark.parametrize("B,Sq,Skv,Hq,Hkv,Dqk,Dv,causal,seed", _random_cases(36, seed=2024))
+def test_random_shapes_match_oracle(gpu, B, Sq, Skv, Hq, Hkv, Dqk, Dv, causal, seed):
+    q, k, v, dout = _inputs(B, Sq, Skv, Hq, Hkv, Dqk, Dv, seed=seed)
+    scale = Dqk**-0.5
+    ref_o, ref_lse = R.chunk_fwd(q, k, v, scale, causal)
+    ref_dq, ref_dk, ref_dv = R.chunk_bwd(q, k, v, dout, ref_lse, R.bwd_delta(ref_o, dout), scale, causal)
+    qd, kd, vd, dod = (t.to(gpu) for t in (q, k, v, dout))
+    o, lse = _mla_fwd(qd, kd, vd, scale, causal=causal)
+    delta = _mla_bwd_preprocess(o, dod)
+    dk, dv = _mla_bwd_dk_dv(qd, kd, vd, dod, lse, delta, scale, causal=causal)
+    dq = _mla_bwd_dq(qd, kd, vd, dod, lse, delta, scale, causal=causal)
+    check_bf16_result(o, ref_o, "O")
+    check_lse(lse, ref_lse, "LSE2")
+    # gradients sum hundreds of bf16-rounded terms: elements much smaller than their row's scale may
+    # miss isclose; allow 0.2 % of them (at least 8 elements of a tiny tensor). The normalised
+    # max-abs and cosine bounds inside check_bf16_result apply to every element.
+    for name, got, want in (("dQ", dq, ref_dq), ("dK", dk, ref_dk), ("dV", dv, ref_dv)):
+        check_bf16_result(got, want, name, otol=max(2e-3, 8.0 / want.numel()))

@@ -52,7 +52,7 @@ struct DkdvLayout {
 // product, ODIM = feature length of the gradient this wave accumulates.
 template <int DQK, int DV, bool CAUSAL, bool ROLE_B, typename Fetch, typename Commit>
 __device__ __forceinline__ void dkdv_wave_loop(const BwdParams& p, char* smem, int lane, int pair, int kv_pair0, int n_iter,
-                                               int n_m, int m_start_wg, const bf16x8* stat,
+                                               int m_end, int m_start_wg, const bf16x8* stat,
                                                f32x16* acc, Fetch& fetch, Commit& commit) {
   using L = DkdvLayout<DQK, DV>;
   constexpr int KDIM = ROLE_B ? DV : DQK;
@@ -66,72 +66,76 @@ __device__ __forceinline__ void dkdv_wave_loop(const BwdParams& p, char* smem, i
   const int m_start_pair = CAUSAL ? kv_pair0 / kBM : 0;
   char* exch = smem + kStages * L::kStage + pair * 8192;
 
+  // Ring stages rotate (prev <- cur <- next <- prev) and the tile position advances by increments:
+  // no division or modulo in the loop. The body has no branch around its matrix instructions (a
+  // tile entirely above this pair's diagonal is processed like any other, its P is all zeros), so
+  // the accumulators stay in place from one iteration to the next.
+  int off_prev = 2 * L::kStage, off_cur = 0, off_next = L::kStage;
+  int mt = m_start_wg;
   for (int i = 0; i < n_iter; ++i) {
-    if (i + 1 < n_iter) commit((i + 1) % kStages);
-    if (i + 2 < n_iter) fetch(i + 2);
-    const char* stage = smem + (i % kStages) * L::kStage;
+    if (i + 1 < n_iter) commit(off_next);
+    if (i + 2 < n_iter) fetch();
+    const char* stage = smem + off_cur;
     const float* stats = reinterpret_cast<const float*>(stage + L::kQTile + L::kOTile);
-    const int mt = m_start_wg + i % n_m;
-    const bool active = mt >= m_start_pair;
     const int q0 = mt * kBM;
 
     f32x16 x;
     bf16x8 frag[2];
-    if (active) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) x[v] = 0.f;
+    for (int v = 0; v < 16; ++v) x[v] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < KDIM / 16; ++ks) {
-        const bf16x8 a = lds_read_straight(stage + T1_OFF, T1P, c, ks * 16 + g * 8);
-        x = mfma32(a, stat[ks], x);
-      }
-      if (!ROLE_B) {
-        // rows of the tile are queries q0 + acc_row(v, g); this lane's column is `key`
-        const bool masked = (CAUSAL && mt == m_start_pair) || (q0 + kBM > p.Sq);
+    for (int ks = 0; ks < KDIM / 16; ++ks) {
+      const bf16x8 a = lds_read_straight(stage + T1_OFF, T1P, c, ks * 16 + g * 8);
+      x = mfma32(a, stat[ks], x);
+    }
+    if (!ROLE_B) {
+      // rows of the tile are queries q0 + acc_row(v, g); this lane's column is `key`
+      f32x4 l4[4];
 #pragma unroll
-        for (int b4 = 0; b4 < 4; ++b4) {
-          const int r0 = 8 * b4 + 4 * g;
-          const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + r0);
-          f32x4 pr;
+      for (int b4 = 0; b4 < 4; ++b4) l4[b4] = *reinterpret_cast<const f32x4*>(stats + 8 * b4 + 4 * g);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float t = __builtin_amdgcn_exp2f(x[4 * b4 + e] * p.kappa - l4[e]);
-            if (masked) {
-              const int qrow = q0 + r0 + e;
-              if ((CAUSAL && key > qrow) || qrow >= p.Sq) t = 0.f;
-            }
-            pr[e] = t;
-            x[4 * b4 + e] = t;
-          }
-          *reinterpret_cast<f32x4*>(exch + (i & 1) * 4096 + (b4 * 64 + lane) * 16) = pr;
+      for (int v = 0; v < 16; ++v) x[v] = __builtin_amdgcn_exp2f(x[v] * p.kappa - l4[v >> 2][v & 3]);
+      if ((CAUSAL && mt <= m_start_pair) || (q0 + kBM > p.Sq)) {  // wave-uniform
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int qrow = q0 + acc_row(v, g);
+          if ((CAUSAL && key > qrow) || qrow >= p.Sq) x[v] = 0.f;
         }
+      }
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) {
+        const f32x4 pr = {x[4 * b4], x[4 * b4 + 1], x[4 * b4 + 2], x[4 * b4 + 3]};
+        *reinterpret_cast<f32x4*>(exch + (i & 1) * 4096 + (b4 * 64 + lane) * 16) = pr;
       }
     }
     __syncthreads();
-    if (active) {
-      if (ROLE_B) {
-        const float* delta_s = stats + kBM;
+    if (ROLE_B) {
+      const float* delta_s = stats + kBM;
+      f32x4 pr[4], d4[4];
 #pragma unroll
-        for (int b4 = 0; b4 < 4; ++b4) {
-          const int r0 = 8 * b4 + 4 * g;
-          const f32x4 pr = *reinterpret_cast<const f32x4*>(exch + (i & 1) * 4096 + (b4 * 64 + lane) * 16);
-          const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_s + r0);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) x[4 * b4 + e] = pr[e] * (x[4 * b4 + e] - d4[e]) * p.scale;
-        }
+      for (int b4 = 0; b4 < 4; ++b4) {
+        pr[b4] = *reinterpret_cast<const f32x4*>(exch + (i & 1) * 4096 + (b4 * 64 + lane) * 16);
+        d4[b4] = *reinterpret_cast<const f32x4*>(delta_s + 8 * b4 + 4 * g);
       }
 #pragma unroll
-      for (int jj = 0; jj < 2; ++jj)
-        frag[jj] = to_bf16x8(x[8 * jj], x[8 * jj + 1], x[8 * jj + 2], x[8 * jj + 3], x[8 * jj + 4], x[8 * jj + 5],
-                             x[8 * jj + 6], x[8 * jj + 7]);
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int o = 0; o < ODIM / 32; ++o) {
-          const bf16x8 a = lds_read_transposed(stage + T2_OFF, T2P, 16 * j, 32 * o, lane);
-          acc[o] = mfma32(a, frag[j], acc[o]);
-        }
+      for (int v = 0; v < 16; ++v) x[v] = pr[v >> 2][v & 3] * (x[v] - d4[v >> 2][v & 3]) * p.scale;
     }
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj)
+      frag[jj] = to_bf16x8(x[8 * jj], x[8 * jj + 1], x[8 * jj + 2], x[8 * jj + 3], x[8 * jj + 4], x[8 * jj + 5],
+                           x[8 * jj + 6], x[8 * jj + 7]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int o = 0; o < ODIM / 32; ++o) {
+        const bf16x8 a = lds_read_transposed(stage + T2_OFF, T2P, 16 * j, 32 * o, lane);
+        acc[o] = mfma32(a, frag[j], acc[o]);
+      }
+    const int t = off_prev;
+    off_prev = off_cur;
+    off_cur = off_next;
+    off_next = t;
+    if (++mt == m_end) mt = m_start_wg;
   }
 }
 
@@ -197,9 +201,13 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
   TileCopy<kBM, DQK, L::QP, kThreads> qcopy;
   TileCopy<kBM, DV, L::OP, kThreads> ocopy;
   float stat_val = 0.f;  // threads 0..31 carry lse, 32..63 carry delta of the tile's rows
-  auto fetch = [&](int it) {
-    const int hq = hq0 + it / n_m;
-    const int mt = m_start_wg + it % n_m;
+  int fetch_hq = hq0, fetch_mt = m_start_wg;  // position of the next tile to fetch
+  auto fetch = [&]() {
+    const int hq = fetch_hq, mt = fetch_mt;
+    if (++fetch_mt == m_tiles_all) {
+      fetch_mt = m_start_wg;
+      ++fetch_hq;
+    }
     qcopy.fetch(p.q + b * p.q_bs + (int64_t)hq * DQK, q_row_stride, mt * kBM, p.Sq, tid);
     ocopy.fetch(p.dout + b * p.dout_bs + (int64_t)hq * DV, do_row_stride, mt * kBM, p.Sq, tid);
     if (tid < 2 * kBM) {
@@ -209,25 +217,25 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
       stat_val = src[row];
     }
   };
-  auto commit = [&](int stage) {
-    char* base = smem + stage * L::kStage;
+  auto commit = [&](int stage_off) {
+    char* base = smem + stage_off;
     qcopy.commit(base, tid);
     ocopy.commit(base + L::kQTile, tid);
     if (tid < 2 * kBM) reinterpret_cast<float*>(base + L::kQTile + L::kOTile)[tid] = stat_val;
   };
 
   if (n_iter > 0) {
-    fetch(0);
+    fetch();
     commit(0);
-    if (n_iter > 1) fetch(1);
+    if (n_iter > 1) fetch();
   }
   wait_all_vector_loads();
   __syncthreads();
 
   if (!role_b)
-    dkdv_wave_loop<DQK, DV, CAUSAL, false>(p, smem, lane, pair, kv_pair0, n_iter, n_m, m_start_wg, stat, acc, fetch, commit);
+    dkdv_wave_loop<DQK, DV, CAUSAL, false>(p, smem, lane, pair, kv_pair0, n_iter, m_tiles_all, m_start_wg, stat, acc, fetch, commit);
   else
-    dkdv_wave_loop<DQK, DV, CAUSAL, true>(p, smem, lane, pair, kv_pair0, n_iter, n_m, m_start_wg, stat, acc, fetch, commit);
+    dkdv_wave_loop<DQK, DV, CAUSAL, true>(p, smem, lane, pair, kv_pair0, n_iter, m_tiles_all, m_start_wg, stat, acc, fetch, commit);
 
   // ---- epilogue: wave A stores dV, wave B stores dK, for key row `key`, features 32*o + 8*b4 + 4*g ..+3
   if (key < p.Skv) {

@@ -73,11 +73,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_bwd_dq_kernel(BwdParams p) {
       for (int v = 0; v < 16; ++v) acc[i][qb][v] = 0.f;
 
   const int n_tiles_all = (p.Skv + BN - 1) / BN;
-  int n_tiles_wg = n_tiles_all, n_tiles_wave = n_tiles_all;
-  if (CAUSAL) {
-    n_tiles_wg = min(n_tiles_all, (m0 + BM - 1) / BN + 1);
-    n_tiles_wave = min(n_tiles_all, (q_wave0 + ROWS_WAVE - 1) / BN + 1);
-  }
+  int n_tiles_wg = n_tiles_all;
+  if (CAUSAL) n_tiles_wg = min(n_tiles_all, (m0 + BM - 1) / BN + 1);
 
   TileCopy<BN, DQK, KP, THREADS> kcopy;
   TileCopy<BN, DV, VP, THREADS> vcopy;
@@ -97,7 +94,10 @@ __global__ __launch_bounds__(WAVES * 64) void attn_bwd_dq_kernel(BwdParams p) {
       vcopy.fetch(vh, v_row_stride, (t + 1) * BN, p.Skv, tid);
     }
 
-    if (t < n_tiles_wave) {
+    // No branch around the matrix instructions: a wave whose rows lie entirely above this tile
+    // under the causal mask processes it like any other (its P is all zeros), which keeps the
+    // accumulators in place across iterations; the workgroup waits for its last wave anyway.
+    {
       f32x16 s[NB][QB], dp[NB][QB];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -126,8 +126,32 @@ __global__ __launch_bounds__(WAVES * 64) void attn_bwd_dq_kernel(BwdParams p) {
         }
 
       const int n0 = t * BN;
-      const bool masked = (CAUSAL && (n0 + BN - 1 > q_wave0)) || (n0 + BN > p.Skv);
+      const bool masked = (CAUSAL && (n0 + BN - 1 > q_wave0)) || (n0 + BN > p.Skv);  // wave-uniform
       bf16x8 dsf[QB][2 * NB];
+      // With registers to spare (small head dims) the mask is a pass of its own under the
+      // wave-uniform branch, which saves a compare and a select per element on unmasked tiles;
+      // at 192/128 that version spills, and the test stays inside the element loop.
+      constexpr bool kMaskPass = DQK + DV <= 192;
+      if (kMaskPass) {
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s[nb][qb][v] = __builtin_amdgcn_exp2f(s[nb][qb][v] * p.kappa - lse_q[qb]);
+        if (masked) {
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) {
+            const int qrow = q_wave0 + qb * 32 + c;
+            const int limit = CAUSAL ? min(qrow, p.Skv - 1) : p.Skv - 1;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+              for (int v = 0; v < 16; ++v)
+                if (n0 + nb * 32 + acc_row(v, g) > limit) s[nb][qb][v] = 0.f;
+          }
+        }
+      }
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const int qrow = q_wave0 + qb * 32 + c;
@@ -136,8 +160,11 @@ __global__ __launch_bounds__(WAVES * 64) void attn_bwd_dq_kernel(BwdParams p) {
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
-            float pr = __builtin_amdgcn_exp2f(s[nb][qb][v] * p.kappa - lse_q[qb]);
-            if (masked && (n0 + nb * 32 + acc_row(v, g) > limit)) pr = 0.f;
+            float pr = s[nb][qb][v];
+            if (!kMaskPass) {
+              pr = __builtin_amdgcn_exp2f(pr * p.kappa - lse_q[qb]);
+              if (masked && (n0 + nb * 32 + acc_row(v, g) > limit)) pr = 0.f;
+            }
             s[nb][qb][v] = pr * (dp[nb][qb][v] - delta_q[qb]) * p.scale;
           }
 #pragma unroll

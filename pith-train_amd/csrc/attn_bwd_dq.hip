@@ -294,8 +294,17 @@ extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t strea
   const BwdParams p = make_bwd_params(a);
   hipStream_t st = (hipStream_t)stream;
   if (a->Dqk == 128) launch_dq<128, 128, 1, 2, 8>(p, a, st);
-  else if (a->Dqk == 192) launch_dq<192, 128, 1, 1, 8>(p, a, st);
-  else launch_dq<64, 64, 1, 1, 8>(p, a, st);
+  else {
+    // short query ranges: workgroups of 4 wavefronts x 32 rows, so that no compute unit idles
+    const bool few = ((a->Sq + 255) / 256) * a->Hq * a->B < 192;
+    if (a->Dqk == 192) {
+      if (few) launch_dq<192, 128, 1, 1, 4>(p, a, st);
+      else launch_dq<192, 128, 1, 1, 8>(p, a, st);
+    } else {
+      if (few) launch_dq<64, 64, 1, 1, 4>(p, a, st);
+      else launch_dq<64, 64, 1, 1, 8>(p, a, st);
+    }
+  }
   return check_launch("pith_attn_bwd_dq");
 }
 

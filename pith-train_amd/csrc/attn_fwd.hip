@@ -245,6 +245,11 @@ void launch_fwd(FwdParams p, const pith_attn_fwd_args* a, hipStream_t st) {
     hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV, false, QB, WAVES>), grid, block, 0, st, p);
 }
 
+// With 256 query rows per workgroup a short query range leaves compute units idle (one workgroup
+// per unit at these LDS sizes): below 3/4 of the device's 256 units the launch uses workgroups
+// of 4 wavefronts x 32 rows instead, which doubles their number.
+bool few_workgroups(int64_t Sq, int64_t Hq, int64_t B) { return ((Sq + 255) / 256) * Hq * B < 192; }
+
 }  // namespace
 }  // namespace pith
 
@@ -280,8 +285,13 @@ extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) 
   p.kappa = a->scale * 1.44269504088896340736f;
   hipStream_t st = (hipStream_t)stream;
   if (a->Dqk == 128 && a->Dv == 128) launch_fwd_d128(p, a->causal != 0, st);
-  else if (a->Dqk == 192 && a->Dv == 128) launch_fwd<192, 128, 1, 8>(p, a, st);
-  else if (a->Dqk == 64 && a->Dv == 64) launch_fwd<64, 64, 1, 8>(p, a, st);
+  else if (a->Dqk == 192 && a->Dv == 128) {
+    if (few_workgroups(a->Sq, a->Hq, a->B)) launch_fwd<192, 128, 1, 4>(p, a, st);
+    else launch_fwd<192, 128, 1, 8>(p, a, st);
+  } else if (a->Dqk == 64 && a->Dv == 64) {
+    if (few_workgroups(a->Sq, a->Hq, a->B)) launch_fwd<64, 64, 1, 4>(p, a, st);
+    else launch_fwd<64, 64, 1, 8>(p, a, st);
+  }
   else
     return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: head dims (Dqk=%lld, Dv=%lld) not in {(64,64),(128,128),(192,128)}",
                 (long long)a->Dqk, (long long)a->Dv);

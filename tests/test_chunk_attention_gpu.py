@@ -47,6 +47,11 @@ CASES = [  # B, Sq, Skv, Hq, Hkv, Dqk, Dv, causal
     pytest.param(1, 193, 193, 8, 1, 128, 128, True, id="d128-193-causal-gqa8"),
     pytest.param(2, 320, 448, 8, 2, 128, 128, False, id="d128-b2-320x448"),
     pytest.param(1, 640, 640, 2, 2, 128, 128, True, id="d128-640-causal"),
+    # enough workgroups for the 8-wavefront variants of the general kernels (shorter query ranges
+    # take the 4-wavefront ones): ceil(Sq/256) * Hq * B >= 192
+    pytest.param(1, 1024, 1024, 48, 48, 192, 128, True, id="mla-h48-s1024-causal-8waves"),
+    pytest.param(1, 1000, 300, 48, 16, 192, 128, False, id="mla-h48-1000x300-8waves"),
+    pytest.param(2, 1536, 1536, 16, 4, 64, 64, True, id="d64-b2-s1536-causal-8waves"),
 ]
 
 

@@ -95,6 +95,30 @@ def zigzag_merge(chunks: Sequence[torch.Tensor], dim: int = 1) -> torch.Tensor:
     return torch.cat(blocks, dim=dim)
 
 
+def cp_local_slice(x: torch.Tensor, cp_rank: int, cp_size: int, layout: str = "contiguous", dim: int = 1) -> torch.Tensor:
+    """The part of a full-sequence tensor (tokens, labels, hidden states) that rank `cp_rank` owns.
+
+    "contiguous" is the reference's slicing (pithtrain/tasks/pretrain_language_model.py:128-133);
+    "zigzag" is what the zigzag ring expects: blocks cp_rank and 2*cp_size-1-cp_rank of 2*cp_size."""
+    assert layout in LAYOUTS, f"layout must be one of {LAYOUTS}, got {layout!r}"
+    n = x.shape[dim]
+    if layout == "contiguous":
+        assert n % cp_size == 0, "sequence length must be a multiple of cp_size"
+        chunk = n // cp_size
+        return x.narrow(dim, cp_rank * chunk, chunk)
+    assert n % (2 * cp_size) == 0, "sequence length must be a multiple of 2 * cp_size"
+    block = n // (2 * cp_size)
+    return torch.cat([x.narrow(dim, cp_rank * block, block), x.narrow(dim, (2 * cp_size - 1 - cp_rank) * block, block)], dim=dim)
+
+
+def cp_position_ids(cp_rank: int, cp_size: int, s_local: int, layout: str = "contiguous", device=None) -> torch.Tensor:
+    """[1, s_local] positions, in the full sequence, of the tokens rank `cp_rank` owns: what the
+    rotary embedding must see. "contiguous" is the reference's offset
+    (pithtrain/models/qwen3_30b_a3b.py:816-821); "zigzag" follows cp_local_slice."""
+    full = torch.arange(cp_size * s_local, device=device).unsqueeze(0)
+    return cp_local_slice(full, cp_rank, cp_size, layout, dim=1)
+
+
 def _rows(t: torch.Tensor, rows: Tuple[int, int]) -> torch.Tensor:
     """Row range of a [B, S, H, D] tensor (a view)."""
     return t if rows == (0, t.shape[1]) else t[:, rows[0] : rows[1]]

@@ -21,8 +21,9 @@ import torch.distributed as dist
 from pithtrain_amd.operators.ring_attention.local import RingBackward, RingForward, ring_schedule
 
 
-def _ring_send_recv_kv(send_k: torch.Tensor, send_v: torch.Tensor, next_global: int, prev_global: int):
-    """Passes the held chunk to the next rank and returns the one arriving from the previous rank."""
+def _post_kv_exchange(send_k: torch.Tensor, send_v: torch.Tensor, next_global: int, prev_global: int):
+    """Starts passing the held chunk to the next rank and receiving the previous rank's chunk.
+    Returns (requests, recv_k, recv_v); the receive buffers are valid after the requests are waited on."""
     assert send_k.is_contiguous() and send_v.is_contiguous(), "ring attention send_k or send_v is not contiguous"
     recv_k, recv_v = torch.empty_like(send_k), torch.empty_like(send_v)
     ops = [
@@ -31,33 +32,51 @@ def _ring_send_recv_kv(send_k: torch.Tensor, send_v: torch.Tensor, next_global: 
         dist.P2POp(dist.irecv, recv_k, prev_global),
         dist.P2POp(dist.irecv, recv_v, prev_global),
     ]
-    for req in dist.batch_isend_irecv(ops):
+    return dist.batch_isend_irecv(ops), recv_k, recv_v
+
+
+def _ring_send_recv_kv(send_k: torch.Tensor, send_v: torch.Tensor, next_global: int, prev_global: int):
+    """Passes the held chunk to the next rank and returns the one arriving from the previous rank
+    (the reference's blocking helper, pithtrain/operators/ring_attention/standard.py:29-50)."""
+    reqs, recv_k, recv_v = _post_kv_exchange(send_k, send_v, next_global, prev_global)
+    for req in reqs:
         req.wait()
     return recv_k, recv_v
 
 
 class RingAttentionDistributedFunc(torch.autograd.Function):
-    """Causal ring attention of one rank inside a context-parallel group (any supported head dims)."""
+    """Causal ring attention of one rank inside a context-parallel group (any supported head dims).
+
+    The exchange of a step is posted BEFORE the step's kernels are enqueued and waited on after
+    them: with the RCCL backend the transfer runs on the communicator's stream while the
+    attention kernels run on the compute stream, so the next chunk (8-25 MB over one xGMI link)
+    arrives behind the current step's compute. The reference waits for each exchange before it
+    computes (standard.py:95-98); the data each step sees is the same."""
 
     @staticmethod
     def forward(ctx, q, k, v, softmax_scale, cp_rank, cp_size, global_ranks, layout="contiguous"):
         assert k.is_contiguous() and v.is_contiguous(), "ring attention k or v is not contiguous"
-        steps = {st.kv_rank: st for st in ring_schedule(cp_rank, cp_size, q.shape[1], layout)}
-        order = [st for st in ring_schedule(cp_rank, cp_size, q.shape[1], layout)]
+        order = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
+        steps = {st.kv_rank: st for st in order}
         fwd = RingForward(q, v.shape[-1], softmax_scale, order, layout)
         next_global = global_ranks[(cp_rank + 1) % cp_size]
         prev_global = global_ranks[(cp_rank - 1) % cp_size]
         cur_k, cur_v = k, v
         saved_k, saved_v, saved_ranks = [], [], []
         for step in range(cp_size):
+            pending = None
+            if step < cp_size - 1:
+                pending = _post_kv_exchange(cur_k, cur_v, next_global, prev_global)
             kv_rank = (cp_rank - step) % cp_size
             if kv_rank in steps:
                 fwd.run_step(steps[kv_rank], cur_k, cur_v)
                 saved_k.append(cur_k)
                 saved_v.append(cur_v)
                 saved_ranks.append(kv_rank)
-            if step < cp_size - 1:
-                cur_k, cur_v = _ring_send_recv_kv(cur_k, cur_v, next_global, prev_global)
+            if pending is not None:
+                reqs, cur_k, cur_v = pending
+                for req in reqs:
+                    req.wait()
         out, lse = fwd.result()
         ctx.save_for_backward(q, out, lse, *saved_k, *saved_v)
         ctx.conf = (softmax_scale, cp_rank, cp_size, list(global_ranks), layout)
@@ -70,39 +89,43 @@ class RingAttentionDistributedFunc(torch.autograd.Function):
         saved = ctx.saved_tensors
         q, out, lse = saved[0], saved[1], saved[2]
         n = len(ctx.saved_ranks)
-        all_k, all_v = list(saved[3 : 3 + n]), list(saved[3 + n : 3 + 2 * n])
+        chunks = {j: (saved[3 + i], saved[3 + n + i]) for i, j in enumerate(ctx.saved_ranks)}
         order = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
+        by_rank = {st.kv_rank: st for st in order}
         bwd = RingBackward(dout, q, out, lse, softmax_scale, order)
-        local_dk = local_dv = None
-        remote_dk, remote_dv = {}, {}
-        for st, k_j, v_j in zip(order, all_k, all_v):
-            dk_j, dv_j = bwd.run_step(st, k_j, v_j)
-            if st.kv_rank == cp_rank:
-                local_dk, local_dv = dk_j, dv_j
-            else:
-                remote_dk[st.kv_rank], remote_dv[st.kv_rank] = dk_j, dv_j
-        dq = bwd.finish()
 
-        wrap = layout == "zigzag"  # every rank visits every chunk, so distances wrap around
+        # Distance 0 is the local chunk. At distance d >= 1 this rank has computed (if the chunk of
+        # rank r-d was visible to it) the gradient that belongs to rank r-d, and rank r+d the one
+        # that belongs here (standard.py:164-187). With the zigzag layout every rank visits every
+        # chunk, so distances wrap around. The exchange of distance d is posted right after the
+        # step that produced its payload and overlaps the next step's kernels; arrivals are added
+        # in order of distance, so the sum does not depend on timing.
+        wrap = layout == "zigzag"
+        local_dk, local_dv = bwd.run_step(by_rank[cp_rank], *chunks[cp_rank])
+        in_flight = []  # (requests, recv_dk, recv_dv, payload kept alive until the send has completed)
         for d in range(1, cp_size):
             target, source = cp_rank - d, cp_rank + d
             if wrap:
                 target, source = target % cp_size, source % cp_size
             ops: List[dist.P2POp] = []
-            recv_dk = recv_dv = None
-            if 0 <= target and target in remote_dk:
-                assert remote_dk[target].is_contiguous() and remote_dv[target].is_contiguous(), (
+            payload = recv_dk = recv_dv = None
+            if 0 <= target and target in by_rank:
+                payload = bwd.run_step(by_rank[target], *chunks[target])
+                assert payload[0].is_contiguous() and payload[1].is_contiguous(), (
                     "ring attention remote_dk or remote_dv is not contiguous"
                 )
-                ops.append(dist.P2POp(dist.isend, remote_dk[target], global_ranks[target]))
-                ops.append(dist.P2POp(dist.isend, remote_dv[target], global_ranks[target]))
+                ops.append(dist.P2POp(dist.isend, payload[0], global_ranks[target]))
+                ops.append(dist.P2POp(dist.isend, payload[1], global_ranks[target]))
             if source < cp_size:
                 recv_dk, recv_dv = torch.empty_like(local_dk), torch.empty_like(local_dv)
                 ops.append(dist.P2POp(dist.irecv, recv_dk, global_ranks[source]))
                 ops.append(dist.P2POp(dist.irecv, recv_dv, global_ranks[source]))
             if ops:
-                for req in dist.batch_isend_irecv(ops):
-                    req.wait()
+                in_flight.append((dist.batch_isend_irecv(ops), recv_dk, recv_dv, payload))
+        dq = bwd.finish()
+        for reqs, recv_dk, recv_dv, _payload in in_flight:
+            for req in reqs:
+                req.wait()
             if recv_dk is not None:
                 local_dk += recv_dk
                 local_dv += recv_dv

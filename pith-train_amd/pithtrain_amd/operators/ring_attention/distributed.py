@@ -54,7 +54,7 @@ class RingAttentionDistributedFunc(torch.autograd.Function):
     computes (standard.py:95-98); the data each step sees is the same."""
 
     @staticmethod
-    def forward(ctx, q, k, v, softmax_scale, cp_rank, cp_size, global_ranks, layout="contiguous"):
+    def forward(ctx, q, k, v, softmax_scale, cp_rank, cp_size, global_ranks, layout="contiguous", rerotate=False):
         assert k.is_contiguous() and v.is_contiguous(), "ring attention k or v is not contiguous"
         order = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
         steps = {st.kv_rank: st for st in order}
@@ -78,9 +78,12 @@ class RingAttentionDistributedFunc(torch.autograd.Function):
                 for req in reqs:
                     req.wait()
         out, lse = fwd.result()
+        if rerotate:  # keep only the local chunk; backward sends the chunks around again
+            saved_k, saved_v, saved_ranks = [k], [v], [cp_rank]
         ctx.save_for_backward(q, out, lse, *saved_k, *saved_v)
         ctx.conf = (softmax_scale, cp_rank, cp_size, list(global_ranks), layout)
         ctx.saved_ranks = saved_ranks
+        ctx.rerotate = rerotate
         return out
 
     @staticmethod
@@ -88,6 +91,10 @@ class RingAttentionDistributedFunc(torch.autograd.Function):
         softmax_scale, cp_rank, cp_size, global_ranks, layout = ctx.conf
         saved = ctx.saved_tensors
         q, out, lse = saved[0], saved[1], saved[2]
+        if ctx.rerotate:
+            dq, dk, dv = _backward_rerotating(dout, q, out, lse, saved[3], saved[4], softmax_scale, cp_rank, cp_size,
+                                              global_ranks, layout)  # fmt: skip
+            return dq, dk, dv, None, None, None, None, None, None
         n = len(ctx.saved_ranks)
         chunks = {j: (saved[3 + i], saved[3 + n + i]) for i, j in enumerate(ctx.saved_ranks)}
         order = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
@@ -129,14 +136,61 @@ class RingAttentionDistributedFunc(torch.autograd.Function):
             if recv_dk is not None:
                 local_dk += recv_dk
                 local_dv += recv_dv
-        return dq, local_dk, local_dv, None, None, None, None, None
+        return dq, local_dk, local_dv, None, None, None, None, None, None
 
 
-def ring_attention_group_func(q, k, v, softmax_scale: float, cp_group, layout: str = "contiguous"):
-    """Resolves rank, size and global ranks of `cp_group` (None = a group of one) and applies the ring."""
+def _backward_rerotating(dout, q, out, lse, k, v, softmax_scale, cp_rank, cp_size, global_ranks, layout):
+    """Backward that keeps one K/V chunk per rank instead of the cp_size chunks the forward saw
+    (the memory cost noted at pithtrain/operators/ring_attention/standard.py:19-21): the chunks
+    go around the ring a second time, each with an fp32 (dK, dV) accumulator travelling beside
+    it. A rank adds its contribution inside the dK/dV kernel's epilogue and passes chunk and
+    accumulator on; after cp_size hops the accumulator is back at the chunk's owner with every
+    rank's share, added in ring order (deterministic). The next K/V chunk is requested before the
+    step's kernels run; the accumulator can only leave after them.
+    Traffic per hop: K, V (bf16) and dK, dV (fp32), against bf16 dK, dV once per remote chunk in
+    the saving variant: memory is traded for link time."""
+    order = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
+    by_rank = {st.kv_rank: st for st in order}
+    bwd = RingBackward(dout, q, out, lse, softmax_scale, order)
+    next_global = global_ranks[(cp_rank + 1) % cp_size]
+    prev_global = global_ranks[(cp_rank - 1) % cp_size]
+    cur_k, cur_v = k, v
+    acc_dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
+    acc_dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
+    for step in range(cp_size):
+        pending_kv = None
+        if step < cp_size - 1:
+            pending_kv = _post_kv_exchange(cur_k, cur_v, next_global, prev_global)
+        kv_rank = (cp_rank - step) % cp_size
+        if kv_rank in by_rank:
+            bwd.run_step(by_rank[kv_rank], cur_k, cur_v, add_to=(acc_dk, acc_dv))
+        if cp_size > 1:
+            recv_dk, recv_dv = torch.empty_like(acc_dk), torch.empty_like(acc_dv)
+            ops = [
+                dist.P2POp(dist.isend, acc_dk, next_global),
+                dist.P2POp(dist.isend, acc_dv, next_global),
+                dist.P2POp(dist.irecv, recv_dk, prev_global),
+                dist.P2POp(dist.irecv, recv_dv, prev_global),
+            ]
+            for req in dist.batch_isend_irecv(ops):
+                req.wait()
+            acc_dk, acc_dv = recv_dk, recv_dv
+        if pending_kv is not None:
+            reqs, cur_k, cur_v = pending_kv
+            for req in reqs:
+                req.wait()
+    dq = bwd.finish()
+    # after cp_size hops the accumulators held here belong to the local chunk
+    return dq, acc_dk.to(k.dtype), acc_dv.to(v.dtype)
+
+
+def ring_attention_group_func(q, k, v, softmax_scale: float, cp_group, layout: str = "contiguous",
+                              rerotate: bool = False):
+    """Resolves rank, size and global ranks of `cp_group` (None = a group of one) and applies the ring.
+    rerotate=True selects the backward that keeps one K/V chunk per rank (_backward_rerotating)."""
     if cp_group is None:
         cp_rank, cp_size, global_ranks = 0, 1, [0]
     else:
         cp_rank, cp_size = cp_group.rank(), cp_group.size()
         global_ranks = [dist.distributed_c10d.get_global_rank(cp_group, r) for r in range(cp_size)]
-    return RingAttentionDistributedFunc.apply(q, k, v, softmax_scale, cp_rank, cp_size, global_ranks, layout)
+    return RingAttentionDistributedFunc.apply(q, k, v, softmax_scale, cp_rank, cp_size, global_ranks, layout, rerotate)

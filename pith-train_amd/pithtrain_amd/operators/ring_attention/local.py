@@ -211,19 +211,27 @@ class RingBackward:
         self.dq_acc = self.dq if single else torch.empty(q.shape, dtype=torch.float32, device=q.device)
         self.done = 0
 
-    def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor):
-        """Returns (dk_j, dv_j), this rank's contribution to chunk st.kv_rank's gradients."""
+    def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor, add_to=None):
+        """Returns (dk_j, dv_j), this rank's contribution to chunk st.kv_rank's gradients.
+
+        With add_to=(dk_acc, dv_acc) (tensors shaped like the chunk, bf16 or fp32) the contribution
+        is ADDED to them inside the kernel epilogue instead, and they are returned: the form a
+        gradient accumulator that travels around the ring with its chunk needs."""
         assert st == self.steps[self.done], "ring steps must be fed in schedule order"
-        dk_j, dv_j = torch.empty_like(k_j), torch.empty_like(v_j)
-        if st.kv_rows != (0, k_j.shape[1]):  # rows of the chunk this rank cannot see get no gradient
-            for t in (dk_j, dv_j):
-                t[:, : st.kv_rows[0]].zero_()
-                t[:, st.kv_rows[1] :].zero_()
+        if add_to is None:
+            dk_j, dv_j = torch.empty_like(k_j), torch.empty_like(v_j)
+            if st.kv_rows != (0, k_j.shape[1]):  # rows of the chunk this rank cannot see get no gradient
+                for t in (dk_j, dv_j):
+                    t[:, : st.kv_rows[0]].zero_()
+                    t[:, st.kv_rows[1] :].zero_()
+        else:
+            dk_j, dv_j = add_to
+            assert dk_j.shape == k_j.shape and dv_j.shape == v_j.shape, "accumulators must be shaped like the chunk"
         qs, ds = _rows(self.q, st.q_rows), _rows(self.dout, st.q_rows)
         ks, vs = _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows)
         ls, dl = _lse_rows(self.lse, st.q_rows), _lse_rows(self.delta, st.q_rows)
         attn_bwd_dkdv_into(qs, ks, vs, ds, ls, dl, _rows(dk_j, st.kv_rows), _rows(dv_j, st.kv_rows),
-                           self.scale, st.causal)  # fmt: skip
+                           self.scale, st.causal, accumulate=add_to is not None)  # fmt: skip
         # Step 0 covers every row and initialises the accumulator; later steps add to their rows.
         attn_bwd_dq_into(qs, ks, vs, ds, ls, dl, _rows(self.dq_acc, st.q_rows), self.scale, st.causal,
                          accumulate=self.done > 0)  # fmt: skip

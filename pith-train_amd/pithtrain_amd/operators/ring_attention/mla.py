@@ -39,9 +39,10 @@ def ring_mla_attention_func(
     cp_group: dist.ProcessGroup,
     *,
     layout: str = "contiguous",
+    rerotate: bool = False,
 ):
     """Causal ring MLA attention across context-parallel ranks."""
-    return ring_attention_group_func(q, k, v, softmax_scale, cp_group, layout)
+    return ring_attention_group_func(q, k, v, softmax_scale, cp_group, layout, rerotate)
 
 
 __all__ = ["ring_mla_attention_func", "RingMLAAttentionFunc", "_online_softmax_combine_log2"]

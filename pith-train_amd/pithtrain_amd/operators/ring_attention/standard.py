@@ -44,10 +44,11 @@ def ring_attention_func(
     cp_group: dist.ProcessGroup,
     *,
     layout: str = "contiguous",
+    rerotate: bool = False,
 ):
     """Causal ring attention across context-parallel ranks."""
     assert q.shape[-1] == v.shape[-1], "ring_attention_func expects equal q/k and v head dims"
-    return ring_attention_group_func(q, k, v, softmax_scale, cp_group, layout)
+    return ring_attention_group_func(q, k, v, softmax_scale, cp_group, layout, rerotate)
 
 
 __all__ = ["ring_attention_func", "RingAttentionFunc", "_online_softmax_combine", "_ring_send_recv_kv"]

@@ -2,7 +2,8 @@
 entry points the driver calls are replaced, inside this test only, by CPU stand-ins built from the
 oracle. What is tested is the part no one-GPU run reaches: which chunk is where at each ring step
 (K/V rotation), which gradients travel back to which rank (distance loop, with and without
-wrap-around), and the reference-named entry points on a real process group. Every rank's O, dQ
+wrap-around; or the accumulator that travels with its chunk in the re-rotating backward), and
+the reference-named entry points on a real process group. Every rank's O, dQ
 and its own chunk's dK/dV must equal full-sequence causal attention restricted to its tokens."""
 
 import socket
@@ -48,7 +49,7 @@ def _install_cpu_stand_ins():
             setattr(L, name, fn)
 
 
-def _worker(rank, world, port, layout, variant, results):
+def _worker(rank, world, port, layout, variant, rerotate, results):
     dist.init_process_group("gloo", init_method=f"tcp://127.0.0.1:{port}", rank=rank, world_size=world)
     try:
         _install_cpu_stand_ins()
@@ -73,7 +74,7 @@ def _worker(rank, world, port, layout, variant, results):
         ql, kl, vl = (mine(t).requires_grad_() for t in (q, k, v))
         group = dist.group.WORLD
         fn = ring_mla_attention_func if variant == "mla" else ring_attention_func
-        out = fn(ql, kl, vl, scale, group, layout=layout)
+        out = fn(ql, kl, vl, scale, group, layout=layout, rerotate=rerotate)
         out.backward(mine(dout))
 
         ro, rl = R.chunk_fwd(q, k, v, scale, True)
@@ -95,14 +96,19 @@ def _free_port():
 
 @pytest.mark.timeout(300)
 @pytest.mark.parametrize(
-    "world,layout,variant",
-    [(2, "contiguous", "gqa"), (2, "zigzag", "gqa"), (3, "zigzag", "mla"), (4, "contiguous", "mla"), (4, "zigzag", "gqa")],
-)
-def test_ring_over_gloo_matches_full_sequence_attention(world, layout, variant):
+    "world,layout,variant,rerotate",
+    [
+        (2, "contiguous", "gqa", False), (2, "zigzag", "gqa", False), (3, "zigzag", "mla", False),
+        (4, "contiguous", "mla", False), (4, "zigzag", "gqa", False),
+        # backward that keeps one K/V chunk per rank and sends the chunks around again
+        (2, "zigzag", "gqa", True), (3, "contiguous", "gqa", True), (4, "zigzag", "mla", True),
+    ],
+)  # fmt: skip
+def test_ring_over_gloo_matches_full_sequence_attention(world, layout, variant, rerotate):
     torch.set_num_threads(1)
     with mp.Manager() as manager:
         results = manager.dict()
-        mp.spawn(_worker, args=(world, _free_port(), layout, variant, results), nprocs=world, join=True)
+        mp.spawn(_worker, args=(world, _free_port(), layout, variant, rerotate, results), nprocs=world, join=True)
         assert sorted(results.keys()) == list(range(world))
         for rank in range(world):
             for name, err in results[rank].items():

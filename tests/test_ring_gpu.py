@@ -104,9 +104,12 @@ def test_zigzag_split_roundtrip():
         assert [c.tolist() for c in zigzag_split(x, C)] == [c.tolist() for c in R.zigzag_split(x, C)]
 
 
-def test_reference_entry_points_with_a_group_of_one(gpu):
+@pytest.mark.parametrize("rerotate", [False, True])
+def test_reference_entry_points_with_a_group_of_one(gpu, rerotate):
     """ring_attention_func / ring_mla_attention_func keep the reference's positional signature;
-    with cp_group=None (a context-parallel group of one) they are plain causal attention."""
+    with cp_group=None (a context-parallel group of one) they are plain causal attention.
+    rerotate=True takes the backward whose dK/dV go through an fp32 accumulator that the kernel
+    adds to (the form that travels around a real ring)."""
     for fn, (H, Hkv, DQ, DV) in ((ring_attention_func, (8, 2, 128, 128)), (ring_mla_attention_func, (4, 4, 192, 128))):
         B, S = 2, 320
         torch.manual_seed(1)
@@ -116,7 +119,7 @@ def test_reference_entry_points_with_a_group_of_one(gpu):
         dout = torch.randn(B, S, H, DV, dtype=torch.bfloat16)
         scale = DQ**-0.5
         qd, kd, vd = (t.to(gpu).requires_grad_(True) for t in (q, k, v))
-        out = fn(qd, kd, vd, scale, None)
+        out = fn(qd, kd, vd, scale, None, rerotate=rerotate)
         out.backward(dout.to(gpu))
         o_ref, lse_ref, dq_ref, dk_ref, dv_ref = _full_reference(q, k, v, dout, scale)
         check_bf16_result(out, o_ref, "O")

@@ -43,6 +43,10 @@ LAYOUT = "zigzag"
 # (`--counter-pass`), scaled by what the same counters read for a plain copy of known size:
 # profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt (215.6 MB read + 67.1 MB written).
 DKDV_TRAFFIC_BYTES = 282_700_000
+# Share of SIMD cycles with the matrix pipe busy over a launch of the roofline kernel, from a
+# rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES / GRBM_GUI_ACTIVE pass over the same `--counter-pass` run
+# (profiles/attn_d128_kernels_mfma_lds_counters.txt); the sustained shader clock there is ~1.87 GHz.
+DKDV_MFMA_BUSY_FRACTION = 0.63
 # The same for the HBM-bound kernels: profiles/combine_norm_rope_mla_assemble_hbm_counters.txt
 COMBINE_TRAFFIC_BYTES = 144_900_000
 NORM_ROPE_TRAFFIC_BYTES = 159_400_000 + 235_200_000  # forward + backward launch
@@ -390,6 +394,7 @@ def main():
             "kernel": "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step)",
             "bound": "mfma", "achieved": round(dkdv_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": DKDV_TRAFFIC_BYTES,
+            "mfma_busy_fraction": DKDV_MFMA_BUSY_FRACTION,
             "ms_per_launch": round(ms_dkdv, 4),
         },  # fmt: skip
         "combine": {

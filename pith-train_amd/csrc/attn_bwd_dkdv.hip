@@ -266,19 +266,30 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
   }
 }
 
-// out[b, s, h, :] (+)= sum over parts of ws[part][b][s][h][:], parts added in index order.
+// out[b, s, h, :] (+)= sum over parts of ws[part][b][s][h][:], parts added in index order; dK
+// (blockIdx.y = 0) and dV (blockIdx.y = 1) in one launch.
+struct ReduceParams {
+  const float* ws[2];
+  void* out[2];
+  int64_t part_stride[2], row_elems[2], out_bs[2], n4[2];
+  int64_t rows_per_batch;
+  int parts, accumulate;
+};
+
 template <typename OutT>
-__global__ __launch_bounds__(256) void reduce_parts_kernel(const float* __restrict__ ws, OutT* out, int parts,
-                                                           int64_t part_stride, int64_t row_elems, int64_t rows_per_batch,
-                                                           int64_t out_bs, int64_t n4, int accumulate) {
+__global__ __launch_bounds__(256) void reduce_parts_kernel(ReduceParams r) {
+  const int t = blockIdx.y;
+  const float* __restrict__ ws = r.ws[t];
+  OutT* out = reinterpret_cast<OutT*>(r.out[t]);
+  const int64_t part_stride = r.part_stride[t], n4 = r.n4[t];
+  const int64_t per_batch = r.rows_per_batch * r.row_elems[t];
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t e = i * 4;
     f32x4 s = *reinterpret_cast<const f32x4*>(ws + e);
-    for (int pidx = 1; pidx < parts; ++pidx) s += *reinterpret_cast<const f32x4*>(ws + pidx * part_stride + e);
-    const int64_t per_batch = rows_per_batch * row_elems;
+    for (int pidx = 1; pidx < r.parts; ++pidx) s += *reinterpret_cast<const f32x4*>(ws + pidx * part_stride + e);
     const int64_t bb = e / per_batch;
-    OutT* dst = out + bb * out_bs + (e - bb * per_batch);
-    store4<OutT>(dst, s[0], s[1], s[2], s[3], accumulate != 0);
+    OutT* dst = out + bb * r.out_bs[t] + (e - bb * per_batch);
+    store4<OutT>(dst, s[0], s[1], s[2], s[3], r.accumulate != 0);
   }
 }
 
@@ -313,23 +324,24 @@ void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
     }
   }
   if (p.split > 1) {
-    const int64_t rows = a->Skv;
+    ReduceParams r;
+    int64_t max_n4 = 0;
     for (int which = 0; which < 2; ++which) {
       const int64_t d = which == 0 ? a->Dqk : a->Dv;
-      const int64_t row_elems = a->Hkv * d;
-      const int64_t part_stride = a->B * rows * row_elems;
-      const int64_t n4 = part_stride / 4;
-      const float* ws = which == 0 ? p.ws_dk : p.ws_dv;
-      void* out = which == 0 ? a->dk : a->dv;
-      const int64_t out_bs = which == 0 ? a->dk_bs : a->dv_bs;
-      const unsigned blocks = (unsigned)((n4 + 255) / 256 < 8192 ? (n4 + 255) / 256 : 8192);
-      if (f32)
-        hipLaunchKernelGGL((reduce_parts_kernel<float>), dim3(blocks), dim3(256), 0, st, ws, (float*)out, p.split,
-                           part_stride, row_elems, rows, out_bs, n4, a->accumulate_dkv);
-      else
-        hipLaunchKernelGGL((reduce_parts_kernel<__bf16>), dim3(blocks), dim3(256), 0, st, ws, (__bf16*)out, p.split,
-                           part_stride, row_elems, rows, out_bs, n4, a->accumulate_dkv);
+      r.row_elems[which] = a->Hkv * d;
+      r.part_stride[which] = a->B * a->Skv * r.row_elems[which];
+      r.n4[which] = r.part_stride[which] / 4;
+      r.ws[which] = which == 0 ? p.ws_dk : p.ws_dv;
+      r.out[which] = which == 0 ? a->dk : a->dv;
+      r.out_bs[which] = which == 0 ? a->dk_bs : a->dv_bs;
+      if (r.n4[which] > max_n4) max_n4 = r.n4[which];
     }
+    r.rows_per_batch = a->Skv;
+    r.parts = p.split;
+    r.accumulate = a->accumulate_dkv;
+    const dim3 rgrid((unsigned)((max_n4 + 255) / 256 < 8192 ? (max_n4 + 255) / 256 : 8192), 2);
+    if (f32) hipLaunchKernelGGL((reduce_parts_kernel<float>), rgrid, dim3(256), 0, st, r);
+    else hipLaunchKernelGGL((reduce_parts_kernel<__bf16>), rgrid, dim3(256), 0, st, r);
   }
 }
 

@@ -6,7 +6,6 @@ import ctypes
 import os
 import re
 import subprocess
-import sys
 
 import pytest
 

@@ -92,7 +92,7 @@ def test_forward_and_backward_match_oracle(gpu, B, Sq, Skv, Hq, Hkv, Dqk, Dv, ca
 
 
 def test_baseline_input_scaling(gpu):
-    """BASELINE inputs are N(0,1)/sqrt(D): outputs are small, so the normalised error is what bites."""
+    """The benchmark inputs are N(0,1)/sqrt(D): outputs are small, so the normalised error is what bites."""
     B, S, Hq, Hkv, D = 1, 1024, 8, 1, 128
     q, k, v, dout = _inputs(B, S, S, Hq, Hkv, D, D, seed=1)
     q, k, v = ((t.float() * D**-0.5).to(torch.bfloat16) for t in (q, k, v))

@@ -143,7 +143,7 @@ def test_cast_f32_bf16_is_round_to_nearest_even(gpu):
 
 
 def test_combine_full_size_properties(gpu):
-    """BASELINE combine shape [1, 4096, 32, 128]: oracle comparison in full (seconds on the CPU),
+    """The benchmark combine shape [1, 4096, 32, 128]: oracle comparison in full (seconds on the CPU),
     commutativity and the identity."""
     o1, l1, o2, l2 = _partials(1, 4096, 32, 128, 42)
     d = [t.to(gpu) for t in (o1, l1, o2, l2)]

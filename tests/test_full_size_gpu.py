@@ -1,4 +1,4 @@
-"""Parity at BASELINE sizes. The dense oracle cannot cover 32K-131K tokens in seconds, so each
+"""Parity at the sizes of the benchmark configurations. The dense oracle cannot cover 32K-131K tokens in seconds, so each
 case runs the whole ring share on the GPU and checks SAMPLED rows against exact full-sequence
 causal attention evaluated only for those rows (cost: rows x total keys):
 
@@ -6,7 +6,7 @@ causal attention evaluated only for those rows (cost: rows x total keys):
   dK_j, dV_j   : sampled key rows of every visited chunk against every local query row, using the
                  kernel's LSE2 and delta (themselves checked on the sampled query rows).
 
-Inputs follow BASELINE's recipe: CPU generator seed 42, q/k/v ~ N(0,1)/sqrt(Dqk), dO ~ N(0,1)."""
+Inputs follow the benchmark recipe: CPU generator seed 42, q/k/v ~ N(0,1)/sqrt(Dqk), dO ~ N(0,1)."""
 
 import pytest
 import torch

@@ -12,10 +12,10 @@
 // into new tensors and a .contiguous(); here every output byte is written once by one kernel and
 // the rotation is evaluated in fp32 with a single rounding.
 //
-// HBM-bound data movement. One thread produces one 16-byte piece of an output tensor: it decodes
-// the piece index into (tensor, head, piece), loads what the piece needs (a straight 16-byte copy,
-// or two input pieces plus cos/sin for a rotated piece) and stores it; consecutive threads write
-// consecutive pieces, so every store of a wavefront is contiguous.
+// HBM-bound data movement. One thread produces 16-byte pieces of the output tensors: it decodes a
+// piece index into (tensor, head, piece), loads what the piece needs (a straight 16-byte copy,
+// or two input pieces plus cos/sin for a rotated piece) and stores it; consecutive threads work
+// on consecutive pieces, so the accesses of a wavefront are contiguous runs.
 #include "pith_common.h"
 
 namespace pith {
@@ -82,39 +82,63 @@ __device__ __forceinline__ void store_piece(__bf16* dst, u32x4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
 }
 
-// Forward. Output pieces of a token, in order: q_out [H][(Dn+Dr)/8], k_out [H][(Dn+Dr)/8], v_out [H][Dv/8].
+constexpr int kBatch = 4;  // copied pieces a thread has in flight
+
+// Forward. A token's output consists of copied pieces (q_nope, k_nope, value: one 16-byte load
+// and store each, issued kBatch loads at a time) and rotated pieces (the rope parts of q_out and,
+// identical for every head, of k_out).
 __global__ __launch_bounds__(kThreads) void mla_assemble_fwd_kernel(AssembleParams p) {
   const int b = blockIdx.y;
   const int64_t s = blockIdx.x;
-  const int qk8 = (p.Dn + p.Dr) >> 3, n8 = p.Dn >> 3, r8 = p.Dr >> 3, v8 = p.Dv >> 3;
-  const int per_qk = p.H * qk8, total = 2 * per_qk + p.H * v8;
+  const int qk = p.Dn + p.Dr, kvw = p.Dn + p.Dv;
+  const int n8 = p.Dn >> 3, r8 = p.Dr >> 3, v8 = p.Dv >> 3;
   const int64_t row = table_row(p, b, s);
-  const __bf16* q = p.q + b * p.q_bs + s * p.H * (int64_t)(p.Dn + p.Dr);
-  const __bf16* kv = p.kv + b * p.kv_bs + s * p.H * (int64_t)(p.Dn + p.Dv);
+  const __bf16* q = p.q + b * p.q_bs + s * p.H * (int64_t)qk;
+  const __bf16* kv = p.kv + b * p.kv_bs + s * p.H * (int64_t)kvw;
   const __bf16* k_pe = p.k_pe + b * p.k_pe_bs + s * p.k_pe_rs;
   const int64_t tok = (int64_t)b * p.S + s;
-  __bf16* q_out = p.q_out + tok * p.H * (p.Dn + p.Dr);
-  __bf16* k_out = p.k_out + tok * p.H * (p.Dn + p.Dr);
+  __bf16* q_out = p.q_out + tok * p.H * qk;
+  __bf16* k_out = p.k_out + tok * p.H * qk;
   __bf16* v_out = p.v_out + tok * p.H * p.Dv;
 
-  for (int o = threadIdx.x; o < total; o += kThreads) {
-    if (o < 2 * per_qk) {
-      const bool is_k = o >= per_qk;
-      const int i = is_k ? o - per_qk : o;
-      const int h = i / qk8, piece = i - h * qk8;
-      __bf16* dst = (is_k ? k_out : q_out) + (int64_t)i * 8;
-      if (piece < n8) {
-        const __bf16* src = is_k ? kv + (int64_t)h * (p.Dn + p.Dv) : q + (int64_t)h * (p.Dn + p.Dr);
-        store_piece(dst, *reinterpret_cast<const u32x4*>(src + 8 * piece));
-      } else {
-        const __bf16* src = is_k ? k_pe : q + (int64_t)h * (p.Dn + p.Dr) + p.Dn;
-        store_piece(dst, rotated_piece(src, p.cos + row, p.sin + row, piece - n8, r8 >> 1));
+  // copied pieces, in order: q_nope [H][Dn/8], k_nope [H][Dn/8], value [H][Dv/8]
+  const int n_nope = p.H * n8, n_copy = 2 * n_nope + p.H * v8;
+  for (int i0 = threadIdx.x; i0 < n_copy; i0 += kThreads * kBatch) {
+    u32x4 val[kBatch];
+    __bf16* dst[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      int i = i0 + u * kThreads;
+      if (i < n_copy) {
+        const __bf16* src;
+        if (i < 2 * n_nope) {
+          const bool is_k = i >= n_nope;
+          i -= is_k ? n_nope : 0;
+          const int h = i / n8, piece = i - h * n8;
+          src = (is_k ? kv + (int64_t)h * kvw : q + (int64_t)h * qk) + 8 * piece;
+          dst[u] = (is_k ? k_out : q_out) + (int64_t)h * qk + 8 * piece;
+        } else {
+          i -= 2 * n_nope;
+          const int h = i / v8, piece = i - h * v8;
+          src = kv + (int64_t)h * kvw + p.Dn + 8 * piece;
+          dst[u] = v_out + (int64_t)i * 8;
+        }
+        val[u] = *reinterpret_cast<const u32x4*>(src);
       }
-    } else {
-      const int i = o - 2 * per_qk;
-      const int h = i / v8, piece = i - h * v8;
-      store_piece(v_out + (int64_t)i * 8, *reinterpret_cast<const u32x4*>(kv + (int64_t)h * (p.Dn + p.Dv) + p.Dn + 8 * piece));
     }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      if (i0 + u * kThreads < n_copy) store_piece(dst[u], val[u]);
+  }
+  // rotated pieces, in order: q_out rope [H][Dr/8], k_out rope [H][Dr/8]
+  const int n_rope = p.H * r8;
+  for (int i = threadIdx.x; i < 2 * n_rope; i += kThreads) {
+    const bool is_k = i >= n_rope;
+    const int j = is_k ? i - n_rope : i;
+    const int h = j / r8, piece = j - h * r8;
+    const __bf16* src = is_k ? k_pe : q + (int64_t)h * qk + p.Dn;
+    __bf16* dst = (is_k ? k_out : q_out) + (int64_t)h * qk + p.Dn + 8 * piece;
+    store_piece(dst, rotated_piece(src, p.cos + row, p.sin + row, piece, r8 >> 1));
   }
 }
 
@@ -148,52 +172,87 @@ __device__ __forceinline__ void load4(const __bf16* src, float* dst, bool add) {
   }
 }
 
-// Backward. Output pieces of a token, in order: dq [H][(Dn+Dr)/8], dkv [H][(Dn+Dv)/8], dk_pe [Dr/8]
-// (dk_pe sums the rope gradient over the heads, in head order, before the inverse rotation).
+// Backward. dk_pe is a sum over all heads: one thread per (head, piece) loads its share of the rope
+// gradient of key_states and leaves it in LDS (all those loads are in flight together), and after
+// the block's other work Dr/8 threads add the heads in head order and apply the inverse rotation.
+// In between: the copied pieces (dq nope from dq_out, dkv nope from dk_out, dkv value from
+// dv_out), kBatch loads at a time, and the rope part of dq.
 __global__ __launch_bounds__(kThreads) void mla_assemble_bwd_kernel(AssembleParams p) {
+  extern __shared__ float rope_grad[];  // [H][Dr/8][8]: (g[4m..4m+3], g[Dr/2+4m..+3]) of every head
   const int b = blockIdx.y;
   const int64_t s = blockIdx.x;
-  const int qk = p.Dn + p.Dr, qk8 = qk >> 3, n8 = p.Dn >> 3, r8 = p.Dr >> 3, kv8 = (p.Dn + p.Dv) >> 3;
+  const int qk = p.Dn + p.Dr, kvw = p.Dn + p.Dv;
+  const int n8 = p.Dn >> 3, r8 = p.Dr >> 3, v8 = p.Dv >> 3;
   const int half = p.Dr >> 1;
-  const int n_dq = p.H * qk8, n_dkv = p.H * kv8, total = n_dq + n_dkv + r8;
   const int64_t row = table_row(p, b, s);
   const int64_t tok = (int64_t)b * p.S + s;
   const __bf16* dq_out = p.dq_out + tok * p.H * qk;
   const __bf16* dk_out = p.dk_out + tok * p.H * qk;
   const __bf16* dv_out = p.dv_out + tok * p.H * p.Dv;
   __bf16* dq = p.q_out + tok * p.H * qk;
-  __bf16* dkv = p.k_out + tok * p.H * (p.Dn + p.Dv);
+  __bf16* dkv = p.k_out + tok * p.H * kvw;
   __bf16* dk_pe = p.v_out + tok * p.Dr;
+  const int n_rope = p.H * r8;
 
-  // walked from the last piece down, so that the few threads with a dk_pe piece (a sum over all
-  // heads) start on it first and the copies that follow hide its latency
-  for (int o = total - 1 - (int)threadIdx.x; o >= 0; o -= kThreads) {
-    if (o < n_dq) {
-      const int h = o / qk8, piece = o - h * qk8;
-      if (piece < n8) {
-        store_piece(dq + (int64_t)o * 8, *reinterpret_cast<const u32x4*>(dq_out + (int64_t)o * 8));
-      } else {
-        const int m = piece - n8;
-        float g_lo[4], g_hi[4];
-        load4(dq_out + (int64_t)h * qk + p.Dn + 4 * m, g_lo, false);
-        load4(dq_out + (int64_t)h * qk + p.Dn + half + 4 * m, g_hi, false);
-        store_piece(dq + (int64_t)o * 8, unrotated_piece(g_lo, g_hi, p.cos + row, p.sin + row, m, half));
+  for (int i = threadIdx.x; i < n_rope; i += kThreads) {
+    const int h = i / r8, m = i - h * r8;
+    float g[8];
+    load4(dk_out + (int64_t)h * qk + p.Dn + 4 * m, g, false);
+    load4(dk_out + (int64_t)h * qk + p.Dn + half + 4 * m, g + 4, false);
+    *reinterpret_cast<f32x4*>(rope_grad + 8 * i) = f32x4{g[0], g[1], g[2], g[3]};
+    *reinterpret_cast<f32x4*>(rope_grad + 8 * i + 4) = f32x4{g[4], g[5], g[6], g[7]};
+  }
+
+  const int n_nope = p.H * n8, n_copy = 2 * n_nope + p.H * v8;
+  for (int i0 = threadIdx.x; i0 < n_copy; i0 += kThreads * kBatch) {
+    u32x4 val[kBatch];
+    __bf16* dst[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      int i = i0 + u * kThreads;
+      if (i < n_copy) {
+        const __bf16* src;
+        if (i < 2 * n_nope) {
+          const bool is_k = i >= n_nope;
+          i -= is_k ? n_nope : 0;
+          const int h = i / n8, piece = i - h * n8;
+          src = (is_k ? dk_out : dq_out) + (int64_t)h * qk + 8 * piece;
+          dst[u] = (is_k ? dkv + (int64_t)h * kvw : dq + (int64_t)h * qk) + 8 * piece;
+        } else {
+          i -= 2 * n_nope;
+          const int h = i / v8, piece = i - h * v8;
+          src = dv_out + (int64_t)i * 8;
+          dst[u] = dkv + (int64_t)h * kvw + p.Dn + 8 * piece;
+        }
+        val[u] = *reinterpret_cast<const u32x4*>(src);
       }
-    } else if (o < n_dq + n_dkv) {
-      const int i = o - n_dq;
-      const int h = i / kv8, piece = i - h * kv8;
-      const __bf16* src = piece < n8 ? dk_out + (int64_t)h * qk + 8 * piece : dv_out + (int64_t)h * p.Dv + 8 * (piece - n8);
-      store_piece(dkv + (int64_t)i * 8, *reinterpret_cast<const u32x4*>(src));
-    } else {
-      const int m = o - n_dq - n_dkv;
-      float g_lo[4] = {0.f, 0.f, 0.f, 0.f}, g_hi[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-      for (int h = 0; h < p.H; ++h) {
-        load4(dk_out + (int64_t)h * qk + p.Dn + 4 * m, g_lo, true);
-        load4(dk_out + (int64_t)h * qk + p.Dn + half + 4 * m, g_hi, true);
-      }
-      store_piece(dk_pe + 8 * m, unrotated_piece(g_lo, g_hi, p.cos + row, p.sin + row, m, half));
     }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      if (i0 + u * kThreads < n_copy) store_piece(dst[u], val[u]);
+  }
+
+  for (int i = threadIdx.x; i < n_rope; i += kThreads) {
+    const int h = i / r8, m = i - h * r8;
+    float g_lo[4], g_hi[4];
+    load4(dq_out + (int64_t)h * qk + p.Dn + 4 * m, g_lo, false);
+    load4(dq_out + (int64_t)h * qk + p.Dn + half + 4 * m, g_hi, false);
+    store_piece(dq + (int64_t)h * qk + p.Dn + 8 * m, unrotated_piece(g_lo, g_hi, p.cos + row, p.sin + row, m, half));
+  }
+
+  __syncthreads();
+  for (int m = threadIdx.x; m < r8; m += kThreads) {
+    float g_lo[4] = {0.f, 0.f, 0.f, 0.f}, g_hi[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < p.H; ++h) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(rope_grad + 8 * (h * r8 + m));
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(rope_grad + 8 * (h * r8 + m) + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        g_lo[e] += lo[e];
+        g_hi[e] += hi[e];
+      }
+    }
+    store_piece(dk_pe + 8 * m, unrotated_piece(g_lo, g_hi, p.cos + row, p.sin + row, m, half));
   }
 }
 
@@ -259,6 +318,9 @@ extern "C" int pith_mla_assemble_fwd(const pith_mla_assemble_args* a, pith_strea
 extern "C" int pith_mla_assemble_bwd(const pith_mla_assemble_args* a, pith_stream_t stream) {
   if (const int rc = validate("pith_mla_assemble_bwd", a, true)) return rc;
   const AssembleParams p = make_params(a);
-  hipLaunchKernelGGL(mla_assemble_bwd_kernel, dim3((unsigned)a->S, (unsigned)a->B), dim3(kThreads), 0, (hipStream_t)stream, p);
+  const size_t lds = (size_t)a->H * a->Dr * sizeof(float);
+  if (lds > 64 * 1024)
+    return fail(PITH_ERR_UNSUPPORTED, "pith_mla_assemble_bwd: H*Dr=%lld exceeds 16384", (long long)(a->H * a->Dr));
+  hipLaunchKernelGGL(mla_assemble_bwd_kernel, dim3((unsigned)a->S, (unsigned)a->B), dim3(kThreads), lds, (hipStream_t)stream, p);
   return check_launch("pith_mla_assemble_bwd");
 }

@@ -216,6 +216,8 @@ def test_mla_assemble_direction_specific_validation():
     assert fwd(ctypes.byref(_mla_assemble_args(k_pe_rs=32)), None) == _C.PITH_ERR_BAD_SHAPE
     assert fwd(ctypes.byref(_mla_assemble_args(k_pe_rs=580)), None) == _C.PITH_ERR_MISALIGNED
     assert fwd(ctypes.byref(_mla_assemble_args(q_bs=1024)), None) == _C.PITH_ERR_BAD_SHAPE
+    # the backward stages every head's rope gradient in LDS: H * Dr is limited
+    assert bwd(ctypes.byref(_mla_assemble_args(H=512)), None) == _C.PITH_ERR_UNSUPPORTED
 
 
 def test_operators_refuse_cpu_tensors():

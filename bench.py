@@ -47,6 +47,7 @@ DKDV_TRAFFIC_BYTES = 282_700_000
 # rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES / GRBM_GUI_ACTIVE pass over the same `--counter-pass` run
 # (profiles/attn_d128_kernels_mfma_lds_counters.txt); the sustained shader clock there is ~1.87 GHz.
 DKDV_MFMA_BUSY_FRACTION = 0.63
+DKDV_SUSTAINED_CLOCK_GHZ = 1.87  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration in the same pass (2.4 GHz nominal)
 # The same for the HBM-bound kernels: profiles/combine_norm_rope_mla_assemble_hbm_counters.txt
 COMBINE_TRAFFIC_BYTES = 144_900_000
 NORM_ROPE_TRAFFIC_BYTES = 159_400_000 + 235_200_000  # forward + backward launch
@@ -394,7 +395,7 @@ def main():
             "kernel": "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step)",
             "bound": "mfma", "achieved": round(dkdv_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": DKDV_TRAFFIC_BYTES,
-            "mfma_busy_fraction": DKDV_MFMA_BUSY_FRACTION,
+            "mfma_busy_fraction": DKDV_MFMA_BUSY_FRACTION, "sustained_clock_ghz": DKDV_SUSTAINED_CLOCK_GHZ,
             "ms_per_launch": round(ms_dkdv, 4),
         },  # fmt: skip
         "combine": {

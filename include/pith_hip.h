@@ -56,6 +56,19 @@ const char* pith_last_error(void);
 /* Symbolic name of an error code ("PITH_OK", "PITH_ERR_BAD_SHAPE", ...). Never NULL. */
 const char* pith_error_name(int code);
 
+/* What the library sees of a device (index as in hipSetDevice): filled from the HIP runtime. The
+ * kernels are built for gfx950 only; `supported` is 1 when arch_name starts with "gfx950". */
+typedef struct {
+  char arch_name[64];
+  int32_t compute_units;
+  int32_t lds_bytes_per_workgroup;
+  int32_t clock_khz;
+  int32_t supported;
+  int64_t hbm_bytes;
+} pith_device_info_t;
+
+int pith_device_info(int device, pith_device_info_t* info);
+
 /* ------------------------------------------------------------------------------------------
  * Online-softmax combine of two partial attention results.
  * Replaces _online_softmax_combine_log2 (ring_attention/mla.py:27-40, base 2) and

@@ -1,6 +1,7 @@
 // Error reporting and version entry points of libpith_hip.so.
 #include <cstdarg>
 #include <cstdio>
+#include <cstring>
 
 #include "pith_common.h"
 
@@ -39,4 +40,19 @@ extern "C" const char* pith_error_name(int code) {
     case PITH_ERR_LAUNCH: return "PITH_ERR_LAUNCH";
     default: return "PITH_ERR_UNKNOWN";
   }
+}
+
+extern "C" int pith_device_info(int device, pith_device_info_t* info) {
+  if (!info) return pith::fail(PITH_ERR_NULL_POINTER, "pith_device_info: info is NULL");
+  hipDeviceProp_t prop;
+  const hipError_t e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess) return pith::fail(PITH_ERR_LAUNCH, "pith_device_info: device %d: %s", device, hipGetErrorString(e));
+  std::memset(info, 0, sizeof(*info));
+  std::strncpy(info->arch_name, prop.gcnArchName, sizeof(info->arch_name) - 1);
+  info->compute_units = prop.multiProcessorCount;
+  info->lds_bytes_per_workgroup = (int32_t)prop.sharedMemPerBlock;
+  info->clock_khz = prop.clockRate;
+  info->supported = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+  info->hbm_bytes = (int64_t)prop.totalGlobalMem;
+  return PITH_OK;
 }

@@ -102,11 +102,19 @@ class MlaAssembleArgs(Structure):
     ]  # fmt: skip
 
 
+class DeviceInfo(Structure):
+    _fields_ = [
+        ("arch_name", ctypes.c_char * 64), ("compute_units", c_int32), ("lds_bytes_per_workgroup", c_int32),
+        ("clock_khz", c_int32), ("supported", c_int32), ("hbm_bytes", c_int64),
+    ]  # fmt: skip
+
+
 # name -> (restype, argtypes); must list every symbol declared in include/pith_hip.h
 SYMBOLS = {
     "pith_version": (c_int, []),
     "pith_last_error": (c_char_p, []),
     "pith_error_name": (c_char_p, [c_int]),
+    "pith_device_info": (c_int, [c_int, POINTER(DeviceInfo)]),
     "pith_combine": (c_int, [POINTER(CombineArgs), c_void_p]),
     "pith_attn_fwd": (c_int, [POINTER(AttnFwdArgs), c_void_p]),
     "pith_attn_bwd_delta": (c_int, [POINTER(AttnDeltaArgs), c_void_p]),
@@ -192,6 +200,6 @@ def bhs_strides(t: torch.Tensor, what: str):
 
 
 __all__ = [
-    "lib", "check", "PithError", "CombineArgs", "AttnFwdArgs", "AttnDeltaArgs", "AttnBwdArgs", "NormRopeArgs", "MlaAssembleArgs", "SYMBOLS",
+    "lib", "check", "PithError", "CombineArgs", "AttnFwdArgs", "AttnDeltaArgs", "AttnBwdArgs", "NormRopeArgs", "MlaAssembleArgs", "DeviceInfo", "SYMBOLS",
     "dtype_code", "current_stream", "require_device", "bshd_batch_stride", "bhs_strides", "byref",
 ]  # fmt: skip

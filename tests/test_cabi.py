@@ -41,6 +41,7 @@ def test_struct_layouts_match_the_header(tmp_path):
         "pith_attn_bwd_args": _C.AttnBwdArgs,
         "pith_norm_rope_args": _C.NormRopeArgs,
         "pith_mla_assemble_args": _C.MlaAssembleArgs,
+        "pith_device_info_t": _C.DeviceInfo,
     }
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "pith_hip.h"', "int main(void){"]
     for cname, st in pairs.items():
@@ -58,6 +59,19 @@ def test_struct_layouts_match_the_header(tmp_path):
         assert int(got[cname]) == ctypes.sizeof(st), cname
         for fname, _ in st._fields_:
             assert int(got[f"{cname}.{fname}"]) == getattr(st, fname).offset, f"{cname}.{fname}"
+
+
+def test_device_info_without_a_device():
+    lib = _C.lib()
+    assert lib.pith_device_info(0, None) == _C.PITH_ERR_NULL_POINTER
+    info = _C.DeviceInfo()
+    rc = lib.pith_device_info(0, ctypes.byref(info))
+    import torch
+
+    if torch.cuda.is_available():
+        assert rc == _C.PITH_OK and info.compute_units > 0
+    else:  # no GPU here: the runtime's error is reported, nothing crashes
+        assert rc == _C.PITH_ERR_LAUNCH and lib.pith_last_error().startswith(b"pith_device_info")
 
 
 def _fwd_args(**kw):

@@ -214,3 +214,49 @@ def test_random_shapes_match_oracle(gpu, B, Sq, Skv, Hq, Hkv, Dqk, Dv, causal, s
     # max-abs and cosine bounds inside check_bf16_result apply to every element.
     for name, got, want in (("dQ", dq, ref_dq), ("dK", dk, ref_dk), ("dV", dv, ref_dv)):
         check_bf16_result(got, want, name, otol=max(2e-3, 8.0 / want.numel()))
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_error_is_within_twice_an_eager_bf16_restatement(gpu, causal):
+    """Inputs at the benchmark scale (N(0,1)/sqrt(D)): the normalised max-abs error of every result
+    against the fp64 oracle is at most twice that of the reference's numerics restated with eager
+    torch ops on the same GPU (fp32 scores from bf16 operands, P and dS rounded to bf16 before
+    the second product, bf16 results)."""
+    from helpers import norm_max_err
+
+    B, S, Hq, Hkv, D = 1, 1024, 8, 2, 128
+    q, k, v, dout = _inputs(B, S, S, Hq, Hkv, D, D, seed=77)
+    q, k, v = ((t.float() * D**-0.5).to(torch.bfloat16) for t in (q, k, v))
+    scale = D**-0.5
+    ref_o, ref_lse = R.chunk_fwd(q, k, v, scale, causal)
+    ref_dq, ref_dk, ref_dv = R.chunk_bwd(q, k, v, dout, ref_lse, R.bwd_delta(ref_o, dout), scale, causal)
+
+    qd, kd, vd, dod = (t.to(gpu) for t in (q, k, v, dout))
+    o, lse = _mla_fwd(qd, kd, vd, scale, causal=causal)
+    delta = _mla_bwd_preprocess(o, dod)
+    dk, dv = _mla_bwd_dk_dv(qd, kd, vd, dod, lse, delta, scale, causal=causal)
+    dq = _mla_bwd_dq(qd, kd, vd, dod, lse, delta, scale, causal=causal)
+
+    # eager restatement, heads first: [B, H, S, D]
+    g = Hq // Hkv
+    qe, doe = qd.transpose(1, 2).float(), dod.transpose(1, 2).float()
+    ke = kd.transpose(1, 2).repeat_interleave(g, dim=1).float()
+    ve = vd.transpose(1, 2).repeat_interleave(g, dim=1).float()
+    s = (qe @ ke.transpose(-1, -2)) * scale
+    if causal:
+        s = s.masked_fill(torch.ones(S, S, dtype=torch.bool, device=gpu).triu(1), float("-inf"))
+    p = torch.softmax(s, dim=-1)
+    p16 = p.to(torch.bfloat16).float()
+    oe = (p16 @ ve).to(torch.bfloat16)
+    de = (oe.float() * doe).sum(-1, keepdim=True)
+    dve = (p16.transpose(-1, -2) @ doe).to(torch.bfloat16)
+    ds16 = (p * (doe @ ve.transpose(-1, -2) - de) * scale).to(torch.bfloat16).float()
+    dqe = (ds16 @ ke).to(torch.bfloat16)
+    dke = (ds16.transpose(-1, -2) @ qe).to(torch.bfloat16)
+    fold = lambda t: t.float().view(B, Hkv, g, S, D).sum(2).to(torch.bfloat16).transpose(1, 2)  # noqa: E731
+    eager = {"O": oe.transpose(1, 2), "dQ": dqe.transpose(1, 2), "dK": fold(dke), "dV": fold(dve)}
+    ours = {"O": o, "dQ": dq, "dK": dk, "dV": dv}
+    want = {"O": ref_o, "dQ": ref_dq, "dK": ref_dk, "dV": ref_dv}
+    for name in ours:
+        e_ours, e_eager = norm_max_err(ours[name], want[name]), norm_max_err(eager[name], want[name])
+        assert e_ours <= 2 * e_eager + 1e-4, f"{name}: error {e_ours:.3e} against {e_eager:.3e} of the eager restatement"

@@ -21,6 +21,12 @@ CASES = [  # Hq, Hkv, Dqk, Dv, S_local, C, rank
     pytest.param(32, 4, 128, 128, 8192, 4, 1, id="qwen3-32k-c4-r1"),
     pytest.param(16, 16, 192, 128, 4096, 4, 1, id="mla-16k-c4-r1"),
     pytest.param(64, 4, 128, 128, 16384, 8, 3, id="long-131k-c8-r3"),
+    # the reference's full-size matrix of the MLA operator, H in {16, 128} x S in {4096, 32768}
+    # (tests/operators/mla/test_triton.py:20-21), as a ring of one: a single causal chunk
+    pytest.param(16, 16, 192, 128, 4096, 1, 0, id="mla-op-h16-s4096"),
+    pytest.param(128, 128, 192, 128, 4096, 1, 0, id="mla-op-h128-s4096"),
+    pytest.param(16, 16, 192, 128, 32768, 1, 0, id="mla-op-h16-s32768"),
+    pytest.param(128, 128, 192, 128, 32768, 1, 0, id="mla-op-h128-s32768"),
 ]
 
 

@@ -182,6 +182,20 @@ int pith_attn_bwd_dq(const pith_attn_bwd_args* args, pith_stream_t stream);
  * workspace is only used during the call's kernels; nothing is kept in it between calls. */
 int64_t pith_attn_bwd_dkdv_workspace_bytes(const pith_attn_bwd_args* args);
 
+/* pith_attn_bwd_dkdv for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the
+ * reference. Same arguments and results, bit for bit, as pith_attn_bwd_dkdv called with a
+ * workspace of pith_attn_bwd_dkdv_workspace_bytes() bytes, but `workspace` / `workspace_bytes`
+ * are ignored: the head-split partial sums go to a scratch array that is part of the library's
+ * code object (PITH_DKDV_STATIC_SCRATCH_BYTES of device memory on every GPU the library runs on,
+ * held until the process ends). The call allocates and frees nothing. A shape whose partial sums
+ * need more than the scratch holds is rejected with PITH_ERR_UNSUPPORTED. The first call on a
+ * device looks up the array's device address (make it outside a graph capture). All calls on
+ * one GPU share that GPU's array: calls that may overlap in time (different streams, different
+ * threads) race and must be ordered by the caller. */
+#define PITH_DKDV_STATIC_SCRATCH_BYTES (64ll << 20)
+int pith_attn_bwd_dkdv_static(const pith_attn_bwd_args* args, pith_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * dst[i] = bf16(src[i]) with round-to-nearest-even, i < n. Replaces the reference's
  * `.to(q.dtype)` on an fp32 accumulator (ring_attention/mla.py:78, standard.py:104) when the

@@ -25,6 +25,8 @@
 // different workgroups (more parallelism when there are few key tiles); the parts leave fp32
 // partial results in a caller-provided workspace and a second kernel adds them in a fixed
 // order, so the result does not depend on scheduling.
+#include <mutex>
+
 #include "attn_bwd_common.h"
 
 namespace pith {
@@ -355,22 +357,81 @@ extern "C" int64_t pith_attn_bwd_dkdv_workspace_bytes(const pith_attn_bwd_args* 
   return workspace_bytes_for(a, pick_split(a));
 }
 
-extern "C" int pith_attn_bwd_dkdv(const pith_attn_bwd_args* a, pith_stream_t stream) {
-  const int rc = validate_bwd(a, "pith_attn_bwd_dkdv", false, true);
-  if (rc != PITH_OK) return rc;
+namespace {
+
+// Runs the kernels with the head-split partials in `workspace` (NULL: no head split).
+int run_dkdv(const pith_attn_bwd_args* a, int split, void* workspace, hipStream_t st, const char* who) {
   BwdParams p = make_bwd_params(a);
-  // Head groups are split only when the caller brought a workspace that is large enough.
-  const int split = pick_split(a);
-  const int64_t need = workspace_bytes_for(a, split);
-  if (split > 1 && a->workspace && a->workspace_bytes >= need) {
-    if (!aligned16(a->workspace)) return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_dkdv: workspace must be 16-byte aligned");
+  if (split > 1 && workspace) {
     p.split = split;
-    p.ws_dk = reinterpret_cast<float*>(a->workspace);
+    p.ws_dk = reinterpret_cast<float*>(workspace);
     p.ws_dv = p.ws_dk + (int64_t)split * a->B * a->Skv * a->Hkv * a->Dqk;
   }
-  hipStream_t st = (hipStream_t)stream;
   if (a->Dqk == 128) launch_dkdv<128, 128>(p, a, st);
   else if (a->Dqk == 192) launch_dkdv<192, 128>(p, a, st);
   else launch_dkdv<64, 64>(p, a, st);
-  return check_launch("pith_attn_bwd_dkdv");
+  return check_launch(who);
+}
+
+// Scratch of pith_attn_bwd_dkdv_static: device memory that belongs to the library's code object
+// (one copy per GPU, held until the process ends). Host code never uses this name as an address;
+// it asks the runtime for the array's device address once per device and passes that on.
+constexpr int64_t kStaticScratchBytes = PITH_DKDV_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device; resolved at the first call on that device.
+int static_scratch(void** out, const char* who) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(PITH_ERR_LAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(PITH_ERR_UNSUPPORTED, "%s: device index %d beyond %d", who, dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(PITH_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", who, dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return PITH_OK;
+}
+
+}  // namespace
+
+extern "C" int pith_attn_bwd_dkdv(const pith_attn_bwd_args* a, pith_stream_t stream) {
+  const int rc = validate_bwd(a, "pith_attn_bwd_dkdv", false, true);
+  if (rc != PITH_OK) return rc;
+  // Head groups are split only when the caller brought a workspace that is large enough.
+  int split = pick_split(a);
+  const int64_t need = workspace_bytes_for(a, split);
+  if (split > 1 && a->workspace && a->workspace_bytes >= need) {
+    if (!aligned16(a->workspace)) return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_dkdv: workspace must be 16-byte aligned");
+  } else {
+    split = 1;
+  }
+  return run_dkdv(a, split, a->workspace, (hipStream_t)stream, "pith_attn_bwd_dkdv");
+}
+
+extern "C" int pith_attn_bwd_dkdv_static(const pith_attn_bwd_args* a, pith_stream_t stream) {
+  const char* who = "pith_attn_bwd_dkdv_static";
+  const int rc = validate_bwd(a, who, false, true);
+  if (rc != PITH_OK) return rc;
+  const int split = pick_split(a);
+  const int64_t need = workspace_bytes_for(a, split);
+  if (need > kStaticScratchBytes)
+    return fail(PITH_ERR_UNSUPPORTED,
+                "%s: the head-split partial sums of this shape need %lld bytes, the built-in scratch holds %lld "
+                "(use pith_attn_bwd_dkdv with a caller-provided workspace)",
+                who, (long long)need, (long long)kStaticScratchBytes);
+  void* ws = nullptr;
+  if (need > 0) {
+    const int src = static_scratch(&ws, who);
+    if (src != PITH_OK) return src;
+  }
+  return run_dkdv(a, split, ws, (hipStream_t)stream, who);
 }

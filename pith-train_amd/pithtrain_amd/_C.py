@@ -120,6 +120,7 @@ SYMBOLS = {
     "pith_attn_bwd_delta": (c_int, [POINTER(AttnDeltaArgs), c_void_p]),
     "pith_attn_bwd_dkdv": (c_int, [POINTER(AttnBwdArgs), c_void_p]),
     "pith_attn_bwd_dq": (c_int, [POINTER(AttnBwdArgs), c_void_p]),
+    "pith_attn_bwd_dkdv_static": (c_int, [POINTER(AttnBwdArgs), c_void_p]),
     "pith_attn_bwd_dkdv_workspace_bytes": (c_int64, [POINTER(AttnBwdArgs)]),
     "pith_cast_f32_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "pith_norm_rope_fwd": (c_int, [POINTER(NormRopeArgs), c_void_p]),

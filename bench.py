@@ -1,25 +1,31 @@
 #!/usr/bin/env python3
 """Benchmark of the ring-attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra-configs]
 
 A step is one forward + backward pass of one GPU's share of causal ring attention at the
 Qwen3-30B-A3B shape (32 q heads / 4 kv heads, head dim 128, 32768 tokens as 4 zigzag chunks of 8192,
 rank 1 of 4): 4 chunk-attention forwards, 3 log2 combines, delta, 4 dK/dV and 4 dQ launches.
-Inputs are synthetic (CPU generator, seed 42; q/k/v ~ N(0,1)/sqrt(128), dO ~ N(0,1)) and resident in
-HBM before the timed region. One JSON line is printed:
+Inputs are synthetic (CPU generator, seed 42; q/k/v ~ N(0,1)/sqrt(Dqk), dO ~ N(0,1)) and resident in
+HBM before the timed region. One JSON line is printed; everything in it is measured in this run
+except the block under "from_profiles", which quotes hardware-counter figures of earlier rocprofv3
+runs by file:
 
   value      algorithmic TFLOP/s of the whole step: 2*(Dqk+Dv)*E*Hq forward + 2*(3Dqk+2Dv)*E*Hq backward
              with E = C*S_l^2/2 score entries per head (5 backward matmuls; recomputation not counted)
+  fwd_only   the forward alone (the forward-only configuration of the same shape)
   roofline   the dominant kernel (non-causal dK/dV), timed per launch with events on the launch stream
+  mla16k     the same ring driver at the MLA shape (16 heads, 192/128, 16384 tokens as 4 zigzag chunks)
+  long131k   the same at the long-context shape (64 q / 4 kv heads, 131072 tokens as 8 zigzag chunks, rank 3)
   combine    the log2 combine at [1,4096,32,128] bf16+bf16 -> fp32 over rotating buffers, GB/s of
-             algorithmic bytes against the 8 TB/s HBM peak, with its own roofline
+             algorithmic bytes against the 8 TB/s HBM peak: timed as replays of a captured HIP graph
+             (kernel time, no host launch cost in between) and, beside it, launched eagerly
   norm_rope  the layer's prologue (per-head RMSNorm + rotary embedding of q [1,8192,32,128] and
              k [1,8192,4,128], forward and backward) over rotating buffers, GB/s of algorithmic bytes
   mla_assemble  the MLA layer's prologue (rotary embedding of the rope parts + assembly of query / key /
              value states, forward and backward) at [1,4096,16,128+64 | 128], GB/s of algorithmic bytes
-  cpu_baseline  the oracle's eager-PyTorch restatement of the same ring share, timed on the host
-             cores over one kv-head group (8 of the 32 query heads)
+  cpu_baseline  the oracle's eager-PyTorch restatement of the same ring share (all heads, once), timed
+             on the host cores
 """
 
 import argparse
@@ -37,40 +43,59 @@ HBM_PEAK_GBPS = 8000.0
 
 HQ, HKV, DQK, DV, S_LOCAL, CP, RANK = 32, 4, 128, 128, 8192, 4, 1
 LAYOUT = "zigzag"
+COMBINE_TRAFFIC = 144_900_000
 
 
-# HBM bytes of one launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes
-# (`--counter-pass`), scaled by what the same counters read for a plain copy of known size:
-# profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt (215.6 MB read + 67.1 MB written).
-DKDV_TRAFFIC_BYTES = 282_700_000
-# Share of SIMD cycles with the matrix pipe busy over a launch of the roofline kernel, from a
-# rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES / GRBM_GUI_ACTIVE pass over the same `--counter-pass` run
-# (profiles/attn_d128_kernels_mfma_lds_counters.txt); the sustained shader clock there is ~1.87 GHz.
-DKDV_MFMA_BUSY_FRACTION = 0.63
-DKDV_SUSTAINED_CLOCK_GHZ = 1.87  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration in the same pass (2.4 GHz nominal)
-# The same for the HBM-bound kernels: profiles/combine_norm_rope_mla_assemble_hbm_counters.txt
-COMBINE_TRAFFIC_BYTES = 144_900_000
-NORM_ROPE_TRAFFIC_BYTES = 159_400_000 + 235_200_000  # forward + backward launch
-MLA_ASSEMBLE_TRAFFIC_BYTES = 128_000_000 + 128_000_000
+# Figures that are NOT measured by this program: hardware-counter results of rocprofv3 --pmc runs over
+# `bench.py --counter-pass`, kept here only so that the JSON line can point at them. They describe the
+# kernels as they were when the named summary was written.
+FROM_PROFILES = {
+    "note": "quoted from committed rocprofv3 summaries, not measured in this run",
+    "attn_bwd_dkdv_d128_kernel<non-causal>": {
+        "file": "profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt",
+        "hbm_bytes_per_launch": 282_700_000,  # 215.6 MB fetched + 67.1 MB written (FETCH_SIZE / WRITE_SIZE, calibrated on a copy)
+        "mfma_file": "profiles/attn_d128_kernels_mfma_lds_counters.txt",
+        "mfma_busy_fraction": 0.63,  # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs)
+        "sustained_clock_ghz": 1.87,  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration (2.4 GHz nominal)
+    },
+    "combine_kernel": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_per_launch": COMBINE_TRAFFIC},
+    "norm_rope_kernels": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_fwd_plus_bwd": 159_400_000 + 235_200_000},
+    "mla_assemble_kernels": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_fwd_plus_bwd": 128_000_000 + 128_000_000},
+}
+
+
+class RingConfig:
+    """One GPU's share of a ring: head counts, head dims, local chunk, ring size, rank (zigzag layout)."""
+
+    def __init__(self, name, hq, hkv, dqk, dv, s_local, cp, rank):
+        self.name, self.hq, self.hkv, self.dqk, self.dv, self.s_local, self.cp, self.rank = name, hq, hkv, dqk, dv, s_local, cp, rank
+
+    def flops(self):
+        entries = self.cp * self.s_local * self.s_local // 2  # per head, this rank's zigzag share
+        return 2 * (self.dqk + self.dv) * entries * self.hq, 2 * (3 * self.dqk + 2 * self.dv) * entries * self.hq
+
+    def make_inputs(self, torch, device, host=False):
+        g = torch.Generator().manual_seed(42)
+        s = self.dqk**-0.5
+        q = (torch.randn(1, self.s_local, self.hq, self.dqk, generator=g) * s).to(torch.bfloat16)
+        ks = [(torch.randn(1, self.s_local, self.hkv, self.dqk, generator=g) * s).to(torch.bfloat16) for _ in range(self.cp)]
+        vs = [(torch.randn(1, self.s_local, self.hkv, self.dv, generator=g) * s).to(torch.bfloat16) for _ in range(self.cp)]
+        dout = torch.randn(1, self.s_local, self.hq, self.dv, generator=g).to(torch.bfloat16)
+        dev = (q.to(device), [c.to(device) for c in ks], [c.to(device) for c in vs], dout.to(device))
+        return ((q, ks, vs, dout) if host else None), dev
+
+
+QWEN3 = RingConfig("qwen3-32k", HQ, HKV, DQK, DV, S_LOCAL, CP, RANK)
+MLA16K = RingConfig("mla-16k", 16, 16, 192, 128, 4096, 4, 1)
+LONG131K = RingConfig("long-131k", 64, 4, 128, 128, 16384, 8, 3)
 
 
 def make_inputs(torch, device):
-    g = torch.Generator().manual_seed(42)
-    s = DQK**-0.5
-    q = (torch.randn(1, S_LOCAL, HQ, DQK, generator=g) * s).to(torch.bfloat16)
-    ks = [(torch.randn(1, S_LOCAL, HKV, DQK, generator=g) * s).to(torch.bfloat16) for _ in range(CP)]
-    vs = [(torch.randn(1, S_LOCAL, HKV, DV, generator=g) * s).to(torch.bfloat16) for _ in range(CP)]
-    dout = torch.randn(1, S_LOCAL, HQ, DV, generator=g).to(torch.bfloat16)
-    host = (q, ks, vs, dout)
-    dev = (q.to(device), [c.to(device) for c in ks], [c.to(device) for c in vs], dout.to(device))
-    return host, dev
+    return QWEN3.make_inputs(torch, device, host=True)
 
 
 def flops_per_step():
-    entries = CP * S_LOCAL * S_LOCAL // 2  # per head, this rank's zigzag share
-    fwd = 2 * (DQK + DV) * entries * HQ
-    bwd = 2 * (3 * DQK + 2 * DV) * entries * HQ
-    return fwd, bwd
+    return QWEN3.flops()
 
 
 def time_events(torch, fn, reps):
@@ -85,41 +110,65 @@ def time_events(torch, fn, reps):
     return start.elapsed_time(stop) / reps
 
 
-def bench_ring(torch, args, dev_inputs):
-    from pithtrain_amd.operators.mla.hip import attn_bwd_dkdv_into
-    from pithtrain_amd.operators.ring_attention.local import (
-        ring_backward_local,
-        ring_forward_local,
-        ring_schedule,
-    )
+def time_ring_share(torch, cfg, dev_inputs, steps, warmup):
+    """(ms per fwd+bwd step by wall clock around synchronised steps, ms forward, ms backward by events)."""
+    from pithtrain_amd.operators.ring_attention.local import ring_backward_local, ring_forward_local
 
     q, ks, vs, dout = dev_inputs
-    scale = DQK**-0.5
+    scale = cfg.dqk**-0.5
 
     def forward():
-        return ring_forward_local(q, ks, vs, scale, RANK, CP, LAYOUT)
+        return ring_forward_local(q, ks, vs, scale, cfg.rank, cfg.cp, LAYOUT)
 
     def step():
         out, lse = forward()
-        return ring_backward_local(dout, q, out, lse, ks, vs, scale, RANK, CP, LAYOUT)
+        return ring_backward_local(dout, q, out, lse, ks, vs, scale, cfg.rank, cfg.cp, LAYOUT)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
-    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    ms_fwd = time_events(torch, forward, args.steps)
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    ms_fwd = time_events(torch, forward, steps)
     out, lse = forward()
-    ms_bwd = time_events(torch, lambda: ring_backward_local(dout, q, out, lse, ks, vs, scale, RANK, CP, LAYOUT), args.steps)
+    ms_bwd = time_events(torch, lambda: ring_backward_local(dout, q, out, lse, ks, vs, scale, cfg.rank, cfg.cp, LAYOUT), steps)
+    return ms_step, ms_fwd, ms_bwd, out, lse
+
+
+def ring_summary(cfg, ms_step, ms_fwd, ms_bwd):
+    fwd_flops, bwd_flops = cfg.flops()
+    tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12  # noqa: E731
+    step_tf = tf(fwd_flops + bwd_flops, ms_step)
+    return {
+        "workload": f"{cfg.hq} q / {cfg.hkv} kv heads, head dims {cfg.dqk}/{cfg.dv}, S={cfg.cp * cfg.s_local} as {cfg.cp} zigzag "
+                    f"chunks of {cfg.s_local} looped locally (rank {cfg.rank}), B=1, fwd+bwd incl. combines and delta",
+        "ms_per_step": round(ms_step, 4), "tflops": round(step_tf, 2), "frac_mfma_peak": round(step_tf / MFMA_BF16_PEAK_TFLOPS, 4),
+        "fwd": {"ms": round(ms_fwd, 4), "tflops": round(tf(fwd_flops, ms_fwd), 2)},
+        "bwd": {"ms": round(ms_bwd, 4), "tflops": round(tf(bwd_flops, ms_bwd), 2)},
+    }  # fmt: skip
+
+
+def bench_other_config(torch, device, cfg, steps, warmup):
+    _, dev = cfg.make_inputs(torch, device)
+    ms_step, ms_fwd, ms_bwd, _, _ = time_ring_share(torch, cfg, dev, steps, warmup)
+    del dev
+    torch.cuda.empty_cache()
+    return ring_summary(cfg, ms_step, ms_fwd, ms_bwd)
+
+
+def bench_ring(torch, args, dev_inputs):
+    from pithtrain_amd.operators.mla.hip import attn_bwd_delta_into, attn_bwd_dkdv_into
+    from pithtrain_amd.operators.ring_attention.local import ring_schedule
+
+    q, ks, vs, dout = dev_inputs
+    scale = DQK**-0.5
+    ms_step, ms_fwd, ms_bwd, out, lse = time_ring_share(torch, QWEN3, dev_inputs, args.steps, args.warmup)
 
     # Dominant kernel: the non-causal dK/dV launch (3 per step; every one covers S_l^2/2 score
     # entries per query head and performs 4 of the 5 algorithmic backward products).
-    from pithtrain_amd.operators.mla.hip import attn_bwd_delta_into
-
     delta = torch.empty_like(lse)
     attn_bwd_delta_into(out, dout, delta)
     st = [s for s in ring_schedule(RANK, CP, S_LOCAL, LAYOUT) if not s.causal]
@@ -157,7 +206,7 @@ def bench_combine(torch, device, reps=50):
     B, S, H, D = 1, 4096, 32, 128
     g = torch.Generator().manual_seed(42)
     sets = []
-    for _ in range(4):  # 4 x 129.5 MiB > the 256 MiB last-level cache
+    for _ in range(5):  # 5 x 129.5 MiB > the 256 MiB last-level cache
         o1 = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(device)
         o2 = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(device)
         l1 = (torch.rand(B, H, S, generator=g) * 16 - 4).to(device)
@@ -174,9 +223,27 @@ def bench_combine(torch, device, reps=50):
 
     for _ in range(8):
         one()
-    ms = time_events(torch, one, reps)
+    ms_eager = time_events(torch, one, reps)
+    # The same rotating sequence captured once in a HIP graph: a replay enqueues the launches back to
+    # back without the host-side cost of each call (the kernel lasts ~25 us, about what the Python
+    # binding spends per call), so the time per launch is the kernel's. The library records no memset
+    # and allocates nothing, which is what makes the capture legal.
+    per_graph = 4 * len(sets)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        one()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    it[0] = 0
+    with torch.cuda.graph(graph):
+        for _ in range(per_graph):
+            one()
+    graph.replay()
+    ms_graph = time_events(torch, graph.replay, max(1, reps // 4)) / per_graph
     host = [t.cpu() for t in sets[0][:4]]
-    return ms, nbytes, host
+    return ms_graph, ms_eager, nbytes, host
 
 
 def bench_norm_rope(torch, device, reps=40):
@@ -285,16 +352,15 @@ def cpu_baseline_norm_rope(torch, host, reps=3):
 
 
 def cpu_baseline_ring(torch, host_inputs):
+    """The whole configuration once on the host cores: every head, every row."""
     from oracle import ring_oracle as R
 
     q, ks, vs, dout = host_inputs
-    heads = (0, HQ // HKV)  # one kv-head group
     t0 = time.perf_counter()
-    R.cpu_ring_fwd_bwd(q, ks, vs, dout, DQK**-0.5, RANK, CP, LAYOUT, heads=heads, q_block=1024)
+    R.cpu_ring_fwd_bwd(q, ks, vs, dout, DQK**-0.5, RANK, CP, LAYOUT, heads=(0, HQ), q_block=1024)
     dt = time.perf_counter() - t0
     fwd, bwd = flops_per_step()
-    sample_flops = (fwd + bwd) * (heads[1] - heads[0]) / HQ
-    return sample_flops / dt / 1e12, dt
+    return (fwd + bwd) / dt / 1e12, dt
 
 
 def cpu_baseline_combine(torch, host, nbytes, reps=5):
@@ -315,6 +381,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra-configs", action="store_true",
+                    help="skip the MLA 16K and long 131K configurations (sub-objects mla16k, long131k)")
     ap.add_argument("--counter-pass", action="store_true",
                     help="run only the roofline kernel and a calibration copy (for rocprofv3 --pmc), print no JSON")
     args = ap.parse_args()
@@ -334,15 +402,21 @@ def main():
     ring = bench_ring(torch, args, dev_inputs)
     if ring is None:
         # the HBM-bound kernels, a few dispatches each, for the same counters
-        bench_combine(torch, device, reps=3)
+        bench_combine(torch, device, reps=4)
         bench_norm_rope(torch, device, reps=3)
         bench_mla_assemble(torch, device, reps=3)
         print("counter pass done")
         return
     ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops = ring
+    del dev_inputs
+    torch.cuda.empty_cache()
     fwd_flops, bwd_flops = flops_per_step()
     tflops = (fwd_flops + bwd_flops) / (ms_step * 1e-3) / 1e12
-    ms_comb, comb_bytes, comb_host = bench_combine(torch, device)
+    mla16k = long131k = None
+    if not args.no_extra_configs:
+        mla16k = bench_other_config(torch, device, MLA16K, args.steps, args.warmup)
+        long131k = bench_other_config(torch, device, LONG131K, max(2, args.steps // 5), 1)
+    ms_comb, ms_comb_eager, comb_bytes, comb_host = bench_combine(torch, device)
     comb_gbps = comb_bytes / (ms_comb * 1e-3) / 1e9
     nr_ms_f, nr_bytes_f, nr_ms_b, nr_bytes_b, nr_host = bench_norm_rope(torch, device)
     nr_gbps = (nr_bytes_f + nr_bytes_b) / ((nr_ms_f + nr_ms_b) * 1e-3) / 1e9
@@ -357,8 +431,8 @@ def main():
         cpu_tflops, cpu_s = cpu_baseline_ring(torch, host_inputs)
         cpu = {
             "value": round(cpu_tflops, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"same workload restricted to one kv-head group (8 of {HQ} query heads), all rows, fp32 eager "
-                      f"PyTorch, {cpu_s:.1f} s; os.cpu_count()={os.cpu_count()}",
+            "sample": f"the whole workload once (all {HQ} query heads, all rows, forward + backward), fp32 eager PyTorch "
+                      f"on bf16-rounded inputs, {cpu_s:.1f} s; os.cpu_count()={os.cpu_count()}",
         }  # fmt: skip
         combine_cpu = {
             "value": round(cpu_baseline_combine(torch, comb_host, comb_bytes), 2), "unit": "GB/s", "cores": cores,
@@ -370,6 +444,7 @@ def main():
         }  # fmt: skip
 
     dkdv_tflops = dkdv_flops / (ms_dkdv * 1e-3) / 1e12
+    dkdv_prof = FROM_PROFILES["attn_bwd_dkdv_d128_kernel<non-causal>"]
     line = {
         "metric": "ring-attn fwd+bwd causal TFLOP/s (Qwen3-30B-A3B, 32K)",
         "value": round(tflops, 2),
@@ -391,19 +466,31 @@ def main():
         "frac_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
         "fwd": {"ms": round(ms_fwd, 4), "tflops": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2)},
         "bwd": {"ms": round(ms_bwd, 4), "tflops": round(bwd_flops / (ms_bwd * 1e-3) / 1e12, 2)},
+        "fwd_only": {
+            "workload": "the same share, forward only (4 chunk-attention launches + 3 combines): O and the base-2 LSE",
+            "ms": round(ms_fwd, 4), "tflops": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2),
+            "frac_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+        },
         "roofline": {
             "kernel": "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step)",
             "bound": "mfma", "achieved": round(dkdv_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": DKDV_TRAFFIC_BYTES,
-            "mfma_busy_fraction": DKDV_MFMA_BUSY_FRACTION, "sustained_clock_ghz": DKDV_SUSTAINED_CLOCK_GHZ,
+            "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+            "traffic": dkdv_prof["hbm_bytes_per_launch"], "traffic_from": dkdv_prof["file"],
             "ms_per_launch": round(ms_dkdv, 4),
         },  # fmt: skip
+        "mla16k": mla16k,
+        "long131k": long131k,
         "combine": {
             "metric": "online_softmax_combine_log2 GB/s ([1,4096,32,128] bf16 x2 -> fp32)",
             "value": round(comb_gbps, 1), "unit": "GB/s", "us_per_launch": round(ms_comb * 1e3, 2),
+            "timing": "replays of a captured HIP graph of 20 launches over 5 rotating buffer sets",
+            "us_per_launch_eager": round(ms_comb_eager * 1e3, 2),
+            "gbps_eager": round(comb_bytes / (ms_comb_eager * 1e-3) / 1e9, 1),
             "bytes": comb_bytes,
             "roofline": {"bound": "hbm", "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": round(comb_gbps / HBM_PEAK_GBPS, 4), "traffic": COMBINE_TRAFFIC_BYTES},
+                         "frac": round(comb_gbps / HBM_PEAK_GBPS, 4),
+                         "traffic": FROM_PROFILES["combine_kernel"]["hbm_bytes_per_launch"],
+                         "traffic_from": FROM_PROFILES["combine_kernel"]["file"]},
             "cpu_baseline": combine_cpu,
         },  # fmt: skip
         "norm_rope": {
@@ -414,7 +501,7 @@ def main():
             "bwd": {"us": round(nr_ms_b * 1e3, 2), "bytes": nr_bytes_b,
                     "gbps": round(nr_bytes_b / (nr_ms_b * 1e-3) / 1e9, 1)},
             "roofline": {"bound": "hbm", "achieved": round(nr_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": round(nr_gbps / HBM_PEAK_GBPS, 4), "traffic": NORM_ROPE_TRAFFIC_BYTES},
+                         "frac": round(nr_gbps / HBM_PEAK_GBPS, 4)},
             "cpu_baseline": norm_rope_cpu,
         },  # fmt: skip
         "mla_assemble": {
@@ -425,8 +512,9 @@ def main():
             "bwd": {"us": round(ma_ms_b * 1e3, 2), "bytes": ma_bytes_b,
                     "gbps": round(ma_bytes_b / (ma_ms_b * 1e-3) / 1e9, 1)},
             "roofline": {"bound": "hbm", "achieved": round(ma_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": round(ma_gbps / HBM_PEAK_GBPS, 4), "traffic": MLA_ASSEMBLE_TRAFFIC_BYTES},
+                         "frac": round(ma_gbps / HBM_PEAK_GBPS, 4)},
         },  # fmt: skip
+        "from_profiles": FROM_PROFILES,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

@@ -1,4 +1,5 @@
 // Error reporting and version entry points of libpith_hip.so.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -17,6 +18,21 @@ int fail(int code, const char* fmt, ...) {
   va_end(ap);
   return code;
 }
+
+int compute_units() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 0) n = 0;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+void begin_launch() { (void)hipGetLastError(); }
 
 int check_launch(const char* what) {
   const hipError_t e = hipGetLastError();

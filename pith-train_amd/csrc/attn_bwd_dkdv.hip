@@ -361,7 +361,12 @@ namespace {
 
 // Runs the kernels with the head-split partials in `workspace` (NULL: no head split).
 int run_dkdv(const pith_attn_bwd_args* a, int split, void* workspace, hipStream_t st, const char* who) {
+  // the grid of this kernel runs over key tiles (validate_bwd bounded the query-side grid)
+  if (((a->Skv + kBN - 1) / kBN) * a->Hkv * a->B * (int64_t)split > 0x7fffffffLL)
+    return fail(PITH_ERR_UNSUPPORTED, "%s: Skv=%lld x Hkv=%lld x B=%lld exceeds the launch grid limit", who,
+                (long long)a->Skv, (long long)a->Hkv, (long long)a->B);
   BwdParams p = make_bwd_params(a);
+  begin_launch();
   if (split > 1 && workspace) {
     p.split = split;
     p.ws_dk = reinterpret_cast<float*>(workspace);

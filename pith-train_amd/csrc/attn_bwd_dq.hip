@@ -293,6 +293,7 @@ extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t strea
   if (rc != PITH_OK) return rc;
   const BwdParams p = make_bwd_params(a);
   hipStream_t st = (hipStream_t)stream;
+  begin_launch();
   if (a->Dqk == 128) launch_dq<128, 128, 1, 2, 8>(p, a, st);
   else {
     // short query ranges: workgroups of 4 wavefronts x 32 rows, so that no compute unit idles

@@ -284,6 +284,7 @@ extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) 
   p.q_bs = a->q_bs; p.k_bs = a->k_bs; p.v_bs = a->v_bs; p.o_bs = a->o_bs; p.lse_bs = a->lse_bs; p.lse_hs = a->lse_hs;
   p.kappa = a->scale * 1.44269504088896340736f;
   hipStream_t st = (hipStream_t)stream;
+  begin_launch();
   if (a->Dqk == 128 && a->Dv == 128) launch_fwd_d128(p, a->causal != 0, st);
   else if (a->Dqk == 192 && a->Dv == 128) {
     if (few_workgroups(a->Sq, a->Hq, a->B)) launch_fwd<192, 128, 1, 4>(p, a, st);

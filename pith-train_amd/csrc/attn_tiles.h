@@ -160,12 +160,17 @@ __device__ __forceinline__ int swizzled_offset(int row, int piece) {
 // Written as inline assembly on purpose: the compiler does not see an LDS write, so it places no
 // wait between this load and later LDS reads of OTHER tiles; the caller waits (s_waitcnt vmcnt)
 // and synchronises the workgroup before anyone reads the destination.
+// The statement overwrites M0 behind the compiler's back: M0 is a reserved register that cannot
+// be declared as clobbered (clang warns that such a declaration is not honoured). That is sound
+// only while the compiler itself emits no M0 use in a kernel that includes this header (dynamic
+// register indexing, s_sendmsg, LDS-DMA or GWS builtins would); tests/test_cabi.py compiles every
+// source to assembly and fails if M0 appears anywhere outside these inline statements.
 __device__ __forceinline__ void load_lds16(const char* base, int offset, char* dst_wave) {
   const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char*)dst_wave;
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(lds_addr), "v"(offset), "s"(base)
-               : "memory");  // m0 is written here and by nothing else in the kernels that use this
+               : "memory");
 }
 
 // 4 bytes per lane from the per-lane global address `src` to LDS at `dst_wave` + 4 * lane (same

@@ -311,6 +311,7 @@ using namespace pith;
 extern "C" int pith_mla_assemble_fwd(const pith_mla_assemble_args* a, pith_stream_t stream) {
   if (const int rc = validate("pith_mla_assemble_fwd", a, false)) return rc;
   const AssembleParams p = make_params(a);
+  begin_launch();
   hipLaunchKernelGGL(mla_assemble_fwd_kernel, dim3((unsigned)a->S, (unsigned)a->B), dim3(kThreads), 0, (hipStream_t)stream, p);
   return check_launch("pith_mla_assemble_fwd");
 }
@@ -321,6 +322,7 @@ extern "C" int pith_mla_assemble_bwd(const pith_mla_assemble_args* a, pith_strea
   const size_t lds = (size_t)a->H * a->Dr * sizeof(float);
   if (lds > 64 * 1024)
     return fail(PITH_ERR_UNSUPPORTED, "pith_mla_assemble_bwd: H*Dr=%lld exceeds 16384", (long long)(a->H * a->Dr));
+  begin_launch();
   hipLaunchKernelGGL(mla_assemble_bwd_kernel, dim3((unsigned)a->S, (unsigned)a->B), dim3(kThreads), lds, (hipStream_t)stream, p);
   return check_launch("pith_mla_assemble_bwd");
 }

@@ -364,8 +364,9 @@ int validate(const char* who, const pith_norm_rope_args* a, bool backward) {
   const int64_t lanes = a->D / 8;
   if (a->D % 8 != 0 || lanes > 64 || (lanes & (lanes - 1)) != 0)
     return fail(PITH_ERR_UNSUPPORTED, "%s: D=%lld must be 8 * a power of two, at most 512", who, (long long)a->D);
-  if (a->B > 65535 || a->H > (1 << 20))
-    return fail(PITH_ERR_UNSUPPORTED, "%s: B=%lld > 65535 or H=%lld > 2^20", who, (long long)a->B, (long long)a->H);
+  if (a->B > 65535 || a->H > (1 << 20) || a->S > (1 << 30))
+    return fail(PITH_ERR_UNSUPPORTED, "%s: B=%lld > 65535, H=%lld > 2^20 or S=%lld > 2^30 (launch grid limits)", who,
+                (long long)a->B, (long long)a->H, (long long)a->S);
   if (a->weight && a->weight_dtype != PITH_BF16 && a->weight_dtype != PITH_F32)
     return fail(PITH_ERR_BAD_DTYPE, "%s: weight dtype %d is not bf16/fp32", who, a->weight_dtype);
   uintptr_t bits = reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->cos) |
@@ -427,7 +428,9 @@ int launch_fwd(const char* who, const pith_norm_rope_args* a, const pith_norm_ro
     pp.t[1] = make_params(b, pb);
     blocks += pb.n_tiles;
   }
+  if (blocks > 0x7fffffffLL) return fail(PITH_ERR_UNSUPPORTED, "%s: %lld row tiles exceed the launch grid limit", who, (long long)blocks);
   const dim3 grid((unsigned)blocks, (unsigned)a->B);
+  begin_launch();
   if (a->weight)
     hipLaunchKernelGGL(norm_rope_fwd_kernel<true>, grid, dim3(kThreads), 0, (hipStream_t)stream, pp);
   else
@@ -466,6 +469,7 @@ int launch_bwd(const char* who, const pith_norm_rope_args* a, const pith_norm_ro
     blocks += pp.t[1].grid_x;
   }
   const dim3 grid((unsigned)blocks, (unsigned)a->B);
+  begin_launch();
   hipStream_t st = (hipStream_t)stream;
   if (!a->weight) {
     hipLaunchKernelGGL(norm_rope_bwd_kernel<false>, grid, dim3(kThreads), 0, st, pp);

@@ -10,8 +10,15 @@ namespace pith {
 
 // Records `msg` (printf-style) as the calling thread's last error and returns `code`.
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
-// Checks hipGetLastError() after a launch; returns PITH_OK or PITH_ERR_LAUNCH.
+// Launch status of an entry point: begin_launch() discards an error an earlier runtime call of
+// the host program may have left behind on this thread (it belongs to that call, and would
+// otherwise be reported against ours); check_launch() then reads the status of the launches made
+// since and returns PITH_OK or PITH_ERR_LAUNCH.
+void begin_launch();
 int check_launch(const char* what);
+
+// Compute units of the current device (looked up once per device; 0 if the runtime cannot tell).
+int compute_units();
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -21,6 +21,7 @@ where q is the q_proj output viewed [b, s, h, dn + dr], kv the kv_b_proj output 
 cos, sin are the rotary module's [positions, dr] tables (bf16); position_ids [b, s] int64 or None.
 """
 
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -35,9 +36,20 @@ def _tables(cos: torch.Tensor, sin: torch.Tensor, dr: int) -> int:
     return cos.shape[0]
 
 
-def _positions(position_ids: Optional[torch.Tensor], b: int, s: int):
+def _positions(position_ids: Optional[torch.Tensor], b: int, s: int, table_rows: int):
+    """Pointer and batch stride of position_ids. The rotary tables must cover every position: the
+    reference indexes them with `cos[position_ids]` (pithtrain/models/deepseek_v2_lite.py:173-187, tables
+    sized at :443-445), which raises on a position beyond the table; the kernel clamps such a position
+    to the table edge to stay inside memory, so a too-short table is rejected here where it can be seen
+    without reading device memory (position_ids=None means positions 0..s-1). With explicit positions the
+    caller sizes the table to max(position_ids)+1 as the reference does; PITHTRAIN_AMD_CHECK_POSITIONS=1
+    adds that check at the price of a device synchronisation."""
     if position_ids is None:
+        assert table_rows >= s, f"rotary tables hold {table_rows} positions, the sequence has {s}"
         return None, 0
+    if os.environ.get("PITHTRAIN_AMD_CHECK_POSITIONS") == "1":
+        lo, hi = int(position_ids.min()), int(position_ids.max())
+        assert 0 <= lo and hi < table_rows, f"position_ids span [{lo}, {hi}], the rotary tables hold {table_rows} positions"
     assert position_ids.dtype == torch.int64, "position_ids must be int64"
     assert position_ids.dim() == 2 and position_ids.shape[0] in (1, b) and position_ids.shape[1] == s, (
         f"position_ids of shape {tuple(position_ids.shape)} does not match [b={b} or 1, s={s}]"
@@ -64,7 +76,8 @@ def mla_assemble_fwd_into(q, kv, k_pe, cos, sin, position_ids, q_out, k_out, v_o
     assert k_pe.stride(2) == 1, "k_pe is not contiguous along its last dim"
     for name, t, shape in (("q_out", q_out, (b, s, h, dqk)), ("k_out", k_out, (b, s, h, dqk)), ("v_out", v_out, (b, s, h, dv))):
         assert t.dtype == torch.bfloat16 and tuple(t.shape) == shape and t.is_contiguous(), f"{name} has the wrong dtype, shape or layout"
-    pos_ptr, pos_bs = _positions(position_ids, b, s)
+    table_rows = _tables(cos, sin, dr)
+    pos_ptr, pos_bs = _positions(position_ids, b, s, table_rows)
     if position_ids is not None:
         _C.require_device(q, position_ids)
     args = _C.MlaAssembleArgs(
@@ -87,7 +100,7 @@ def mla_assemble_bwd_into(dq_out, dk_out, dv_out, cos, sin, position_ids, dq, dk
                            ("dv_out", dv_out, (b, s, h, dv)), ("dq", dq, (b, s, h, dqk)),
                            ("dkv", dkv, (b, s, h, dn + dv)), ("dk_pe", dk_pe, (b, s, dr))):  # fmt: skip
         assert t.dtype == torch.bfloat16 and tuple(t.shape) == shape and t.is_contiguous(), f"{name} has the wrong dtype, shape or layout"
-    pos_ptr, pos_bs = _positions(position_ids, b, s)
+    pos_ptr, pos_bs = _positions(position_ids, b, s, _tables(cos, sin, dr))
     args = _C.MlaAssembleArgs(
         q=None, kv=None, k_pe=None, cos=cos.data_ptr(), sin=sin.data_ptr(), position_ids=pos_ptr,
         q_out=dq.data_ptr(), k_out=dkv.data_ptr(), v_out=dk_pe.data_ptr(),

@@ -272,3 +272,37 @@ def test_ring_schedule_matches_oracle_schedule():
             for r in range(C):
                 ours = [(s.kv_rank, s.causal, s.q_rows, s.kv_rows) for s in ring_schedule(r, C, 64, layout)]
                 assert ours == R._steps(r, C, 64, layout)
+
+
+def test_m0_is_touched_only_by_the_direct_load_statements(tmp_path):
+    """csrc/attn_tiles.h sets M0 inside inline assembly (the LDS destination of global_load_lds), which
+    the compiler cannot be told about. Compile every kernel source to gfx950 assembly and check that
+    no instruction OUTSIDE the inline-assembly regions (;;#ASMSTART ... ;;#ASMEND) mentions M0, i.e. that the
+    compiler keeps no M0 state of its own that those statements could corrupt."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    from pithtrain_amd import build as B
+
+    def offending(src):
+        out = tmp_path / (src + ".s")
+        cmd = [B._hipcc(), *B.HIPCC_FLAGS, "-I", B.INCLUDE_DIR, "-I", B.SRC_DIR, "--cuda-device-only", "-S",
+               os.path.join(B.SRC_DIR, src), "-o", str(out)]  # fmt: skip
+        subprocess.run(cmd, check=True, capture_output=True)
+        bad, in_asm = [], False
+        for line in out.read_text().splitlines():
+            code = line.split(";")[0]
+            if "#ASMSTART" in line:
+                in_asm = True
+            elif "#ASMEND" in line:
+                in_asm = False
+            elif not in_asm and re.search(r"\bm0\b", code):
+                bad.append(f"{src}: {line.strip()}")
+        return bad
+
+    users = [s for s in B.SOURCES if "attn_tiles.h" in open(os.path.join(B.SRC_DIR, s)).read()
+             or "attn_bwd_common.h" in open(os.path.join(B.SRC_DIR, s)).read()
+             or "attn_fwd_common.h" in open(os.path.join(B.SRC_DIR, s)).read()]  # fmt: skip
+    assert users
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        bad = [b for res in pool.map(offending, users) for b in res]
+    assert not bad, "compiler-generated M0 use next to inline M0 writes:\n" + "\n".join(bad[:10])

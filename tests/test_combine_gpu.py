@@ -133,6 +133,48 @@ def test_combine_row_range_in_place_and_bf16_out(gpu):
     ).all()
 
 
+@pytest.mark.parametrize("dts", [("bf16", "bf16", "f32"), ("bf16", "bf16", "bf16"), ("f32", "bf16", "f32"),
+                                 ("f32", "bf16", "bf16"), ("bf16", "f32", "f32"), ("f32", "f32", "f32")])
+@pytest.mark.parametrize("B,S,H,D", [
+    (1, 96, 32, 128),   # fp32 chunks: 32 rows x 32 chunks = 256 x 4 per position
+    (2, 40, 64, 128),   # 64 heads: 256 x 8 (the long-context shape)
+    (1, 64, 16, 128),   # 16 heads (MLA): two positions per tile
+    (1, 24, 8, 64),     # 8 positions per tile
+    (1, 1000, 32, 128),  # more tiles than one round of blocks covers on a 256-CU device, ragged last round
+])
+def test_combine_front_walk_equals_per_tile_kernel(gpu, dts, B, S, H, D):
+    """Shapes that take the front-walking kernel (one block per compute unit, tiles of 256 x U chunks) in
+    every dtype combination and unroll, in place and out of place, against the oracle, and bit for bit
+    against the per-tile kernel: the same problem with one position appended no longer divides into
+    front tiles evenly (S odd -> one position per tile is still possible, so a head is appended instead:
+    H+1 heads never give 256 x U chunks) and is served by the per-tile kernel."""
+    dt = {"bf16": torch.bfloat16, "f32": torch.float32}
+    d1, d2, do = (dt[x] for x in dts)
+    o1, l1, o2, l2 = _partials(B, S, H + 1, D, 31, d1, d2)
+    # per-tile kernel on H+1 heads, then compare heads [0, H)
+    big = [t.to(gpu) for t in (o1, l1, o2, l2)]
+    out_big = torch.empty(B, S, H + 1, D, dtype=do, device=gpu)
+    lse_big = torch.empty(B, H + 1, S, dtype=torch.float32, device=gpu)
+    combine_into(*big, out_big, lse_big)
+    small = [o1[:, :, :H].contiguous().to(gpu), l1[:, :H].contiguous().to(gpu),
+             o2[:, :, :H].contiguous().to(gpu), l2[:, :H].contiguous().to(gpu)]  # fmt: skip
+    out = torch.full((B, S, H, D), float("nan"), dtype=do, device=gpu)
+    lse = torch.full((B, H, S), float("nan"), dtype=torch.float32, device=gpu)
+    combine_into(*small, out, lse)
+    assert torch.equal(out, out_big[:, :, :H]) and torch.equal(lse, lse_big[:, :H])
+    ro, rl = R.combine_log2(small[0].double().cpu(), small[1].double().cpu(), small[2].double().cpu(), small[3].double().cpu())
+    if do == torch.float32:
+        assert_close(out, ro, rtol=2e-6, atol=2e-6, what="combined out")
+    else:
+        assert_close(out, ro, rtol=2**-8 * 1.01, atol=1e-6, what="combined out (bf16)")  # one rounding to bf16: half an ulp
+    check_lse(lse, rl, "combined lse", tol=1e-5)
+    # in place: out aliases the partial of its dtype, lse_out aliases lse1
+    if do in (d1, d2):
+        tgt = small[0] if do == d1 else small[2]
+        combine_into(*small, tgt, small[1])
+        assert torch.equal(tgt, out) and torch.equal(small[1], lse)
+
+
 def test_cast_f32_bf16_is_round_to_nearest_even(gpu):
     g = torch.Generator().manual_seed(0)
     x = torch.randn(4096, generator=g) * 100

@@ -126,3 +126,40 @@ def test_reference_entry_points_with_a_group_of_one(gpu, rerotate):
         check_bf16_result(qd.grad, dq_ref, "dQ", otol=1e-3)
         check_bf16_result(kd.grad, dk_ref, "dK", otol=1e-3)
         check_bf16_result(vd.grad, dv_ref, "dV", otol=1e-3)
+
+
+@pytest.fixture
+def one_rank_group(tmp_path):
+    """A real torch.distributed ProcessGroup with a single member (file rendezvous, gloo): the object the
+    model code hands to ring_attention_func. A ring of one issues no collective."""
+    import torch.distributed as dist
+
+    assert not dist.is_initialized()
+    dist.init_process_group("gloo", init_method=f"file://{tmp_path}/rendezvous", rank=0, world_size=1)
+    try:
+        yield dist.new_group([0])
+    finally:
+        dist.destroy_process_group()
+
+
+def test_reference_entry_points_with_a_process_group(gpu, one_rank_group):
+    """Positional call exactly as the reference's layers make it (qwen3_30b_a3b.py:432-438,
+    deepseek_v2_lite.py:456-465): ring_attention_func(q, k, v, softmax_scale, cp_group) with a
+    ProcessGroup object, so that cp_group.rank() / size() / get_global_rank are exercised on the GPU path."""
+    assert one_rank_group.size() == 1 and one_rank_group.rank() == 0
+    for fn, (H, Hkv, DQ, DV) in ((ring_attention_func, (8, 2, 128, 128)), (ring_mla_attention_func, (4, 4, 192, 128))):
+        B, S = 1, 384
+        torch.manual_seed(3)
+        q = torch.randn(B, S, H, DQ, dtype=torch.bfloat16)
+        k = torch.randn(B, S, Hkv, DQ, dtype=torch.bfloat16)
+        v = torch.randn(B, S, Hkv, DV, dtype=torch.bfloat16)
+        dout = torch.randn(B, S, H, DV, dtype=torch.bfloat16)
+        scale = DQ**-0.5
+        qd, kd, vd = (t.to(gpu).requires_grad_(True) for t in (q, k, v))
+        out = fn(qd, kd, vd, scale, one_rank_group)
+        out.backward(dout.to(gpu))
+        o_ref, lse_ref, dq_ref, dk_ref, dv_ref = _full_reference(q, k, v, dout, scale)
+        check_bf16_result(out, o_ref, "O")
+        check_bf16_result(qd.grad, dq_ref, "dQ", otol=1e-3)
+        check_bf16_result(kd.grad, dk_ref, "dK", otol=1e-3)
+        check_bf16_result(vd.grad, dv_ref, "dV", otol=1e-3)

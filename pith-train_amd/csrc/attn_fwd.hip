@@ -245,6 +245,19 @@ void launch_fwd(FwdParams p, const pith_attn_fwd_args* a, hipStream_t st) {
     hipLaunchKernelGGL((attn_fwd_kernel<DQK, DV, false, QB, WAVES>), grid, block, 0, st, p);
 }
 
+// Work split of the direct-load kernels: 256-row workgroups (one per compute unit at a time) unless
+// they would leave the device badly used; then 128-row workgroups, twice as many, each about a
+// fifth less efficient. Under the causal mask the heaviest workgroup carries twice the average
+// work, so a launch needs about four rounds of workgroups before the light ones fill the gaps;
+// without a mask only the fill of the last round matters.
+bool prefer_half_rows(int64_t Sq, int64_t Hq, int64_t B, bool causal) {
+  const int64_t cus = compute_units() > 0 ? compute_units() : 256;
+  const int64_t wgs = ((Sq + 255) / 256) * Hq * B;
+  if (causal) return wgs < 4 * cus;
+  const int64_t rounds = (wgs + cus - 1) / cus;
+  return wgs * 4 < rounds * cus * 3;  // less than 3/4 of the slots of its rounds
+}
+
 // With 256 query rows per workgroup a short query range leaves compute units idle (one workgroup
 // per unit at these LDS sizes): below 3/4 of the device's 256 units the launch uses workgroups
 // of 4 wavefronts x 32 rows instead, which doubles their number.
@@ -285,10 +298,8 @@ extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) 
   p.kappa = a->scale * 1.44269504088896340736f;
   hipStream_t st = (hipStream_t)stream;
   begin_launch();
-  if (a->Dqk == 128 && a->Dv == 128) launch_fwd_d128(p, a->causal != 0, st);
-  else if (a->Dqk == 192 && a->Dv == 128) {
-    if (few_workgroups(a->Sq, a->Hq, a->B)) launch_fwd<192, 128, 1, 4>(p, a, st);
-    else launch_fwd<192, 128, 1, 8>(p, a, st);
+  if ((a->Dqk == 128 || a->Dqk == 192) && a->Dv == 128) {
+    launch_fwd_direct(p, (int)a->Dqk, a->causal != 0, prefer_half_rows(a->Sq, a->Hq, a->B, a->causal != 0), st);
   } else if (a->Dqk == 64 && a->Dv == 64) {
     if (few_workgroups(a->Sq, a->Hq, a->B)) launch_fwd<64, 64, 1, 4>(p, a, st);
     else launch_fwd<64, 64, 1, 8>(p, a, st);

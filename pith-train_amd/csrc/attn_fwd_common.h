@@ -20,7 +20,9 @@ struct FwdParams {
   float kappa;  // scale * log2(e)
 };
 
-// Forward for head dims (128, 128): attn_fwd_d128.hip.
-void launch_fwd_d128(FwdParams p, bool causal, hipStream_t stream);
+// Forward for head dims (128, 128) and (192, 128) with tiles loaded global -> LDS directly:
+// attn_fwd_direct.hip. dqk = 128 or 192; half = workgroups of 128 query rows whose wave pairs split
+// the keys of every tile (see there) instead of 256-row workgroups.
+void launch_fwd_direct(const FwdParams& p, int dqk, bool causal, bool half, hipStream_t stream);
 
 }  // namespace pith

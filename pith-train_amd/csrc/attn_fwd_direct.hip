@@ -1,8 +1,8 @@
-// Chunk attention forward for head dims (128, 128) on gfx950. Same function and numerics as the
-// general kernel in attn_fwd.hip (pithtrain/operators/mla/triton.py:32-93, :274-323: fp32
-// scores from bf16 MFMA, P = exp2(kappa*(s - m)) in fp32, row sum from the fp32 P, P rounded to
-// bf16 for P V, base-2 LSE, lazily refreshed running maximum), organised around two facts
-// measured on the device:
+// Chunk attention forward for head dims (128, 128) and (192, 128) on gfx950. Same function and
+// numerics as the general kernel in attn_fwd.hip (pithtrain/operators/mla/triton.py:32-93,
+// :274-323: fp32 scores from bf16 MFMA, P = exp2(kappa*(s - m)) in fp32, row sum from the fp32 P,
+// P rounded to bf16 for P V, base-2 LSE, lazily refreshed running maximum), organised around two
+// facts measured on the device:
 //   - the two wavefronts that share a SIMD overlap matrix and vector work only while they are in
 //     DIFFERENT phases; left alone they fall into lock step (both in MFMA, then both in VALU);
 //   - moving K/V tiles through registers into LDS costs several hundred cycles per tile of
@@ -14,6 +14,19 @@
 // [P = softmax(S)]; early waves run matrix then vector, late waves vector then matrix, so on
 // each SIMD one wave's MFMAs coincide with the other's softmax. In its matrix block a wave has
 // no help in hiding LDS latency, so the fragment reads run a few products ahead of their use.
+//
+// Head dim 192 (the MLA key: 128 + 64 features): a K tile is the packed 128-feature tile plus a
+// second packed tile for features 128..191 that holds TWO keys per 256-byte row (key r in pieces
+// 0-7, key r+32 in pieces 8-15 of row r), so that both are read with the same conflict-free
+// swizzle.
+//
+// Two work splits. FULL: a workgroup owns 256 query rows, a wave 32 of them and all 64 keys of
+// every tile. HALF: a workgroup owns 128 query rows; the two waves of a SIMD own the SAME 32 rows,
+// the early one keys 0-31 and the late one keys 32-63 of every tile, each with its own running
+// maximum, sum and accumulator, merged through LDS at the end. HALF doubles the number of
+// workgroups (for launches that would leave compute units idle or badly balanced under the
+// causal mask) and halves the registers per wave that depend on the tile width, at the price of
+// half as many matrix instructions between two barriers.
 #include <type_traits>
 
 #include "attn_fwd_common.h"
@@ -23,41 +36,67 @@ namespace {
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
-constexpr int kBM = kWaves * 32;  // query rows per workgroup
 constexpr int kBN = kFwdBlockN;   // keys per tile
-constexpr int kD = 128;
+constexpr int kDv = 128;
 constexpr int kDist = 2;   // a tile is requested kDist intervals before the interval that reads it
 constexpr int kSlots = 4;  // ring depth per operand, > kDist; a power of two (the slot index is a mask)
 static_assert(kSlots > kDist && (kSlots & (kSlots - 1)) == 0, "ring depth");
 constexpr int kAhead = 4;  // fragment reads run this many products ahead in the matrix block
-constexpr int kTile = kBN * kRowBytes128;
+constexpr int kTile = kBN * kRowBytes128;          // a packed 128-feature tile of 64 rows
+constexpr int kExtraTile = kBN / 2 * kRowBytes128;  // features 128..191 of 64 keys, two keys per row
 
-template <bool CAUSAL>
-__global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
-  constexpr int KS = kD / 16;   // contraction steps of Q K^T
-  constexpr int DVB = kD / 32;  // 32-row blocks of O^T
-  __shared__ __attribute__((aligned(1024))) char smem[2 * kSlots * kTile];
+// Moves features 128..191 of a 64-key tile into the two-keys-per-row packed tile: one
+// global_load_lds per thread of a 512-thread workgroup (wave w fills rows 4w .. 4w+3).
+struct DirectExtra64 {
+  int src_off, row_bytes;
+  __device__ __forceinline__ static int source(int row_bytes, int wave, int lane, int rows_left) {
+    const int row = 4 * wave + (lane >> 4);
+    const int piece = (lane & 15) ^ tile_swizzle(row);
+    int key = row + 32 * (piece >> 3);
+    key = key < rows_left ? key : rows_left - 1;
+    return key * row_bytes + 256 + ((piece & 7) << 4);
+  }
+  __device__ __forceinline__ void init(int row_bytes_, int wave, int lane) {
+    row_bytes = row_bytes_;
+    src_off = source(row_bytes_, wave, lane, kBN);
+  }
+  __device__ __forceinline__ void issue(const char* tile_src, int rows_left, char* slot, int wave, int lane) const {
+    if (rows_left >= kBN) load_lds16(tile_src, src_off, slot + wave * 1024);
+    else load_lds16(tile_src, source(row_bytes, wave, lane, rows_left), slot + wave * 1024);
+  }
+};
+
+template <int DQK, bool HALF, bool CAUSAL>
+__global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) {
+  constexpr int KS = DQK / 16;    // contraction steps of Q K^T
+  constexpr int DVB = kDv / 32;   // 32-row blocks of O^T
+  constexpr int KVB = HALF ? 1 : 2;          // 32-key blocks of a tile this wave owns
+  constexpr int kBM = HALF ? 128 : 256;      // query rows per workgroup
+  constexpr int kKTile = kTile + (DQK == 192 ? kExtraTile : 0);
+  static_assert(DQK == 128 || DQK == 192, "head dims");
+  __shared__ __attribute__((aligned(1024))) char smem[kSlots * (kKTile + kTile)];
   char* const kbuf = smem;
-  char* const vbuf = smem + kSlots * kTile;
+  char* const vbuf = smem + kSlots * kKTile;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, g = lane >> 5;
   const bool late = wave >= kWaves / 2;  // shares its SIMD with wave - kWaves/2
+  const int kvb0 = HALF ? (wave >> 2) : 0;  // first 32-key block of a tile this wave owns
 
   int m_tile, h, b;
   decode_block(blockIdx.x, p.Hq, p.B, p.m_tiles, m_tile, h, b);
   const int hk = h / p.group;
   const int m0 = m_tile * kBM;
-  const int q_wave0 = m0 + wave * 32;
+  const int q_wave0 = m0 + (HALF ? (wave & 3) : wave) * 32;
   const int qrow = q_wave0 + c;
 
-  const int64_t q_row_stride = (int64_t)p.Hq * kD;
-  const int64_t o_row_stride = (int64_t)p.Hq * kD;
-  const int kv_row_bytes = p.Hkv * kD * 2;
-  const __bf16* qh = p.q + b * p.q_bs + (int64_t)h * kD;
-  const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * kD);
-  const char* vh = reinterpret_cast<const char*>(p.v + b * p.v_bs + (int64_t)hk * kD);
+  const int64_t q_row_stride = (int64_t)p.Hq * DQK;
+  const int64_t o_row_stride = (int64_t)p.Hq * kDv;
+  const int k_row_bytes = p.Hkv * DQK * 2, v_row_bytes = p.Hkv * kDv * 2;
+  const __bf16* qh = p.q + b * p.q_bs + (int64_t)h * DQK;
+  const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * DQK);
+  const char* vh = reinterpret_cast<const char*>(p.v + b * p.v_bs + (int64_t)hk * kDv);
 
   // Number of key tiles this workgroup / this wavefront has to visit.
   const int n_tiles_all = (p.Skv + kBN - 1) / kBN;
@@ -67,13 +106,25 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
     n_tiles_wave = min(n_tiles_all, (q_wave0 + 31) / kBN + 1);
   }
 
-  DirectTile128<kBN, kThreads> mover;
-  mover.init(kv_row_bytes, wave, lane);
+  DirectTile128<kBN, kThreads> mover, kmover;  // V tiles (and K tiles when the row pitches agree); K tiles otherwise
+  DirectExtra64 xmover;
+  mover.init(v_row_bytes, wave, lane);
+  if constexpr (DQK != kDv) {
+    kmover.init(k_row_bytes, wave, lane);
+    xmover.init(k_row_bytes, wave, lane);
+  }
   auto issue_k = [&](int t) __attribute__((always_inline)) {
-    mover.issue(kh + (int64_t)t * kBN * kv_row_bytes, p.Skv - t * kBN, kbuf + (t & (kSlots - 1)) * kTile, wave, lane);
+    char* slot = kbuf + (t & (kSlots - 1)) * kKTile;
+    const char* src = kh + (int64_t)t * kBN * k_row_bytes;
+    if constexpr (DQK != kDv) {
+      kmover.issue(src, p.Skv - t * kBN, slot, wave, lane);
+      xmover.issue(src, p.Skv - t * kBN, slot + kTile, wave, lane);
+    } else {
+      mover.issue(src, p.Skv - t * kBN, slot, wave, lane);
+    }
   };
   auto issue_v = [&](int t) __attribute__((always_inline)) {
-    mover.issue(vh + (int64_t)t * kBN * kv_row_bytes, p.Skv - t * kBN, vbuf + (t & (kSlots - 1)) * kTile, wave, lane);
+    mover.issue(vh + (int64_t)t * kBN * v_row_bytes, p.Skv - t * kBN, vbuf + (t & (kSlots - 1)) * kTile, wave, lane);
   };
   // tiles needed by the prologue (K 0), interval 0 (K 1, V 0) and interval 1 (K 2, V 1)
   issue_k(0);
@@ -93,14 +144,25 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
   }
 
   // per-lane read offsets inside a tile
-  int k_off[KS];      // straight fragment of key row c, contraction step ks (+ 32 rows: + 8192 bytes)
+  // k_off[ks]: straight fragment of this wave's first key block, row c, contraction step ks. Steps
+  // 0..7 lie in the 128-feature tile (the next key block: + 32 rows = + 8192 bytes); steps 8.. in
+  // the extra tile behind it, whose row c holds key c in pieces 0-7 and key c + 32 in pieces 8-15
+  // (the next key block: piece + 8, i.e. the offset with bit 7 flipped).
+  int k_off[KS];
   int v_off[DVB][2];  // transposing reads of feature block i, lower / upper 8 keys (+ 16 keys: + 4096 bytes)
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) k_off[ks] = straight_offset128(c, 2 * ks + g);
+  for (int ks = 0; ks < KS; ++ks) {
+    if (ks < 8) k_off[ks] = straight_offset128(c, 2 * ks + g) + kvb0 * 32 * kRowBytes128;
+    else k_off[ks] = kTile + straight_offset128(c, 2 * (ks - 8) + g + 8 * kvb0);
+  }
+  auto k_frag = [&](const char* ktile, int ks, int kvb) __attribute__((always_inline)) {
+    const int off = ks < 8 ? k_off[ks] + kvb * 32 * kRowBytes128 : (kvb ? k_off[ks] ^ 128 : k_off[ks]);
+    return *reinterpret_cast<const bf16x8*>(ktile + off);
+  };
 #pragma unroll
   for (int i = 0; i < DVB; ++i)
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh) v_off[i][hh] = transposed_offset128(0, hh, 32 * i, lane);
+    for (int hh = 0; hh < 2; ++hh) v_off[i][hh] = transposed_offset128(0, hh, 32 * i, lane) + kvb0 * 32 * kRowBytes128;
 
   f32x16 oacc[DVB];
 #pragma unroll
@@ -110,22 +172,19 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
   float m_run = -INFINITY;
   float l_run = 0.f;  // this lane's share of the row sum (the partner lane holds the rest)
 
-  f32x16 s[2];   // S^T of one key tile: [64 keys] x [32 queries] as two 32 x 32 tiles
-  bf16x8 pf[4];  // P^T of one key tile as B operand, one fragment per 16 keys
+  f32x16 s[KVB];       // S^T of this wave's keys of one tile: 32 x 32 tiles [keys] x [queries]
+  bf16x8 pf[2 * KVB];  // P^T of the same keys as B operand, one fragment per 16 keys
 
   // ---- S^T = K Q^T
   auto scores = [&](const char* ktile) __attribute__((always_inline)) {
 #pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
+    for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) s[kvb][v] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(ktile + k_off[ks] + kvb * 32 * kRowBytes128);
-        s[kvb] = mfma32(a, qf[ks], s[kvb]);
-      }
+      for (int kvb = 0; kvb < KVB; ++kvb) s[kvb] = mfma32(k_frag(ktile, ks, kvb), qf[ks], s[kvb]);
   };
 
   // ---- mask, online softmax (one query column per lane pair), P^T fragments
@@ -135,16 +194,16 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
       // tile crossing the diagonal of a causal chunk, or a ragged last tile
       const int limit = CAUSAL ? min(qrow, p.Skv - 1) : p.Skv - 1;  // last visible key
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb)
+      for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int key = n0 + kvb * 32 + acc_row(v, g);
+          const int key = n0 + (kvb0 + kvb) * 32 + acc_row(v, g);
           if (key > limit) s[kvb][v] = -INFINITY;
         }
     }
     float x = s[0][0];
 #pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
+    for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) x = fmaxf(x, s[kvb][v]);
     const float mx = pair_max(x);
@@ -163,7 +222,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
     const float mk = (m_run == -INFINITY) ? 0.f : m_run * p.kappa;
     float rs = 0.f;
 #pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
+    for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const float e = __builtin_amdgcn_exp2f(s[kvb][v] * p.kappa - mk);
@@ -172,7 +231,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
       }
     l_run += rs;
 #pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
+    for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
       for (int jj = 0; jj < 2; ++jj) {
         const f32x16& x16 = s[kvb];
@@ -184,7 +243,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
   // ---- O^T += V^T P^T
   auto accumulate = [&](const char* vtile) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2 * KVB; ++j)
 #pragma unroll
       for (int i = 0; i < DVB; ++i) {
         const bf16x8 a = lds_read_transposed_at(vtile + v_off[i][0] + j * 16 * kRowBytes128,
@@ -196,10 +255,11 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
   // ---- matrix block of one interval: O^T += V^T P^T of one tile, then S^T of the next, with
   // the fragment reads pinned kAhead products ahead of their use.
   auto matrix_block = [&](const char* vtile, const char* ktile) __attribute__((always_inline)) {
-    constexpr int NPV = 4 * DVB, NQK = 2 * KS;
-    bf16x8 av[4][DVB], ak[KS][2];
+    constexpr int NPV = 2 * KVB * DVB, NQK = KVB * KS;
+    static_assert(kAhead <= NPV, "look-ahead assumes it starts inside the P V product");
+    bf16x8 av[2 * KVB][DVB], ak[KS][KVB];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2 * KVB; ++j)
 #pragma unroll
       for (int i = 0; i < DVB; ++i)
         av[j][i] = lds_read_transposed_at(vtile + v_off[i][0] + j * 16 * kRowBytes128,
@@ -207,20 +267,19 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb)
-        ak[ks][kvb] = *reinterpret_cast<const bf16x8*>(ktile + k_off[ks] + kvb * 32 * kRowBytes128);
+      for (int kvb = 0; kvb < KVB; ++kvb) ak[ks][kvb] = k_frag(ktile, ks, kvb);
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2 * KVB; ++j)
 #pragma unroll
       for (int i = 0; i < DVB; ++i) oacc[i] = mfma32(av[j][i], pf[j], oacc[i]);
 #pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
+    for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) s[kvb][v] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb) s[kvb] = mfma32(ak[ks][kvb], qf[ks], s[kvb]);
+      for (int kvb = 0; kvb < KVB; ++kvb) s[kvb] = mfma32(ak[ks][kvb], qf[ks], s[kvb]);
     // a transposed fragment takes two LDS reads, a straight one a single read
     __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
 #pragma unroll
@@ -238,7 +297,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
 
   // Every interval ends by waiting until at most the loads of the last kDist - 1 intervals are
   // still in flight (the tiles of the next interval have landed), and a workgroup barrier.
-  constexpr int kPerInterval = 2 * DirectTile128<kBN, kThreads>::kPerThread;
+  constexpr int kPerInterval = 2 * DirectTile128<kBN, kThreads>::kPerThread + (DQK == 192 ? 1 : 0);
   static_assert((kDist - 1) * kPerInterval < 16, "vmcnt immediate below assumes a 4-bit low field");
   auto land_and_sync = [&](bool steady) __attribute__((always_inline)) {
     if (steady) __builtin_amdgcn_s_waitcnt(0x0F70 | ((kDist - 1) * kPerInterval));
@@ -257,7 +316,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
   auto interval = [&](int i, auto late_tag, auto full_tag) __attribute__((always_inline)) {
     constexpr bool LATE = decltype(late_tag)::value, FULL = decltype(full_tag)::value;
     const char* vtile = vbuf + (i & (kSlots - 1)) * kTile;
-    const char* ktile = kbuf + ((i + 1) & (kSlots - 1)) * kTile;
+    const char* ktile = kbuf + ((i + 1) & (kSlots - 1)) * kKTile;
     const bool steady = i + 1 + kDist < n_tiles_wg;  // both a K and a V tile are requested in this interval
     // Requests are placed where no LDS read of the same wave follows closely: after the matrix
     // block in the early waves, before the vector block in the late ones.
@@ -296,8 +355,44 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
     for (; i < n_tiles_wg; ++i) interval(i, std::true_type{}, std::false_type{});
   }
 
+  // ---- HALF: the late wave of a pair hands its accumulator, maximum and sum to the early wave,
+  // which rescales both to the common maximum and adds them. The tile ring is free by now (every
+  // wave passed the barrier that ends the last interval).
+  if constexpr (HALF) {
+    constexpr int kExch = 16 * 64 * 16 + 64 * 8;  // 64 accumulator values and (m, l) per lane
+    char* const exch = smem + (wave & 3) * kExch;
+    if (late) {
+#pragma unroll
+      for (int i = 0; i < DVB; ++i)
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          const f32x4 v4 = {oacc[i][4 * b4], oacc[i][4 * b4 + 1], oacc[i][4 * b4 + 2], oacc[i][4 * b4 + 3]};
+          *reinterpret_cast<f32x4*>(exch + ((i * 4 + b4) * 64 + lane) * 16) = v4;
+        }
+      const f32x2 ml = {m_run, l_run};
+      *reinterpret_cast<f32x2*>(exch + 16 * 64 * 16 + lane * 8) = ml;
+    }
+    __syncthreads();
+    if (late) return;
+    const f32x2 ml = *reinterpret_cast<const f32x2*>(exch + 16 * 64 * 16 + lane * 8);
+    const float m_new = fmaxf(m_run, ml[0]);
+    // a side that saw no key has m = -inf, l = 0 and a zero accumulator: weight 0
+    const float a_e = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m_new) * p.kappa);
+    const float a_l = (ml[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((ml[0] - m_new) * p.kappa);
+    m_run = m_new;
+    l_run = l_run * a_e + ml[1] * a_l;
+#pragma unroll
+    for (int i = 0; i < DVB; ++i)
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) {
+        const f32x4 v4 = *reinterpret_cast<const f32x4*>(exch + ((i * 4 + b4) * 64 + lane) * 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) oacc[i][4 * b4 + e] = oacc[i][4 * b4 + e] * a_e + v4[e] * a_l;
+      }
+  }
+
   // ---- epilogue: normalise, store O (bf16) and LSE2
-  __bf16* oh = p.o + b * p.o_bs + (int64_t)h * kD;
+  __bf16* oh = p.o + b * p.o_bs + (int64_t)h * kDv;
   float* lse = p.lse + b * p.lse_bs + (int64_t)h * p.lse_hs;
   const float l = pair_sum(l_run);
   const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -316,15 +411,25 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_d128_kernel(FwdParams p) {
   }
 }
 
-}  // namespace
-
-void launch_fwd_d128(FwdParams p, bool causal, hipStream_t st) {
+template <int DQK, bool HALF>
+void launch_one(FwdParams p, bool causal, hipStream_t st) {
+  constexpr int kBM = HALF ? 128 : 256;
   p.m_tiles = (p.Sq + kBM - 1) / kBM;
   const dim3 grid((unsigned)(p.m_tiles * p.Hq * p.B)), block(kThreads);
-  if (causal)
-    hipLaunchKernelGGL((attn_fwd_d128_kernel<true>), grid, block, 0, st, p);
-  else
-    hipLaunchKernelGGL((attn_fwd_d128_kernel<false>), grid, block, 0, st, p);
+  if (causal) hipLaunchKernelGGL((attn_fwd_direct_kernel<DQK, HALF, true>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((attn_fwd_direct_kernel<DQK, HALF, false>), grid, block, 0, st, p);
+}
+
+}  // namespace
+
+void launch_fwd_direct(const FwdParams& p, int dqk, bool causal, bool half, hipStream_t st) {
+  if (dqk == 128) {
+    if (half) launch_one<128, true>(p, causal, st);
+    else launch_one<128, false>(p, causal, st);
+  } else {
+    if (half) launch_one<192, true>(p, causal, st);
+    else launch_one<192, false>(p, causal, st);
+  }
 }
 
 }  // namespace pith

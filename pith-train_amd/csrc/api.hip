@@ -32,6 +32,19 @@ int compute_units() {
   return n;
 }
 
+// Work split of the direct-load kernels: 256-row workgroups (one per compute unit at a time) unless
+// they would leave the device badly used; then 128-row workgroups, twice as many, each about a
+// fifth less efficient. Under the causal mask the heaviest workgroup carries twice the average
+// work, so a launch needs about four rounds of workgroups before the light ones fill the gaps;
+// without a mask only the fill of the last round matters.
+bool prefer_half_rows(int64_t Sq, int64_t Hq, int64_t B, bool causal) {
+  const int64_t cus = compute_units() > 0 ? compute_units() : 256;
+  const int64_t wgs = ((Sq + 255) / 256) * Hq * B;
+  if (causal) return wgs < 4 * cus;
+  const int64_t rounds = (wgs + cus - 1) / cus;
+  return wgs * 4 < rounds * cus * 3;  // less than 3/4 of the slots of its rounds
+}
+
 void begin_launch() { (void)hipGetLastError(); }
 
 int check_launch(const char* what) {

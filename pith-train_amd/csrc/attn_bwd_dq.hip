@@ -294,17 +294,22 @@ extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t strea
   const BwdParams p = make_bwd_params(a);
   hipStream_t st = (hipStream_t)stream;
   begin_launch();
-  if (a->Dqk == 128) launch_dq<128, 128, 1, 2, 8>(p, a, st);
-  else {
+  const bool half = prefer_half_rows(a->Sq, a->Hq, a->B, a->causal != 0);
+  if ((a->Dqk == 128 && half) || a->Dqk == 192) {
+    // 128-row workgroups whose wave pairs split every tile's keys: the only direct-load form for
+    // 192-feature queries, and the better one for 128 features when 256-row workgroups would
+    // leave compute units idle
+    BwdParams q = p;
+    q.tiles = (int)((a->Sq + 127) / 128);
+    q.accumulate = a->accumulate_dq;
+    launch_dq_direct(q, (int)a->Dqk, a->causal != 0, a->dq_dtype == PITH_F32, st);
+  } else if (a->Dqk == 128) {
+    launch_dq<128, 128, 1, 2, 8>(p, a, st);
+  } else {
     // short query ranges: workgroups of 4 wavefronts x 32 rows, so that no compute unit idles
     const bool few = ((a->Sq + 255) / 256) * a->Hq * a->B < 192;
-    if (a->Dqk == 192) {
-      if (few) launch_dq<192, 128, 1, 1, 4>(p, a, st);
-      else launch_dq<192, 128, 1, 1, 8>(p, a, st);
-    } else {
-      if (few) launch_dq<64, 64, 1, 1, 4>(p, a, st);
-      else launch_dq<64, 64, 1, 1, 8>(p, a, st);
-    }
+    if (few) launch_dq<64, 64, 1, 1, 4>(p, a, st);
+    else launch_dq<64, 64, 1, 1, 8>(p, a, st);
   }
   return check_launch("pith_attn_bwd_dq");
 }

@@ -42,29 +42,8 @@ constexpr int kDist = 2;   // a tile is requested kDist intervals before the int
 constexpr int kSlots = 4;  // ring depth per operand, > kDist; a power of two (the slot index is a mask)
 static_assert(kSlots > kDist && (kSlots & (kSlots - 1)) == 0, "ring depth");
 constexpr int kAhead = 4;  // fragment reads run this many products ahead in the matrix block
-constexpr int kTile = kBN * kRowBytes128;          // a packed 128-feature tile of 64 rows
-constexpr int kExtraTile = kBN / 2 * kRowBytes128;  // features 128..191 of 64 keys, two keys per row
-
-// Moves features 128..191 of a 64-key tile into the two-keys-per-row packed tile: one
-// global_load_lds per thread of a 512-thread workgroup (wave w fills rows 4w .. 4w+3).
-struct DirectExtra64 {
-  int src_off, row_bytes;
-  __device__ __forceinline__ static int source(int row_bytes, int wave, int lane, int rows_left) {
-    const int row = 4 * wave + (lane >> 4);
-    const int piece = (lane & 15) ^ tile_swizzle(row);
-    int key = row + 32 * (piece >> 3);
-    key = key < rows_left ? key : rows_left - 1;
-    return key * row_bytes + 256 + ((piece & 7) << 4);
-  }
-  __device__ __forceinline__ void init(int row_bytes_, int wave, int lane) {
-    row_bytes = row_bytes_;
-    src_off = source(row_bytes_, wave, lane, kBN);
-  }
-  __device__ __forceinline__ void issue(const char* tile_src, int rows_left, char* slot, int wave, int lane) const {
-    if (rows_left >= kBN) load_lds16(tile_src, src_off, slot + wave * 1024);
-    else load_lds16(tile_src, source(row_bytes, wave, lane, rows_left), slot + wave * 1024);
-  }
-};
+constexpr int kTile = kBN * kRowBytes128;  // a packed 128-feature tile of 64 rows
+constexpr int kExtraTile = kExtraTileBytes;  // features 128..191 of 64 keys, two keys per row
 
 template <int DQK, bool HALF, bool CAUSAL>
 __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) {

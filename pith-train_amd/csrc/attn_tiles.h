@@ -222,6 +222,36 @@ struct DirectTile128 {
   }
 };
 
+// ---------------------------------------------------------------------------------------------
+// Features 128..191 of a 64-row tile of a 192-feature operand (the MLA key / query): a second
+// packed tile that holds TWO tile rows per 256-byte LDS row, row r in pieces 0-7 and row r + 32
+// in pieces 8-15 of LDS row r (r < 32), under the same swizzle. Read like a 32-row, 128-feature
+// tile whose features 64..127 are the second 32-row block: a straight fragment of row block kb,
+// row c, contraction step x (0..3) is piece 2x + g + 8*kb of LDS row c; a transposed fragment of
+// row block kb, feature block f (0..1) uses col_base = 64*kb + 32*f.
+constexpr int kExtraTileBytes = 32 * kRowBytes128;
+
+// Moves that part of a tile global memory -> LDS: one global_load_lds per thread of a 512-thread
+// workgroup (wave w fills LDS rows 4w .. 4w+3). Source rows are 384 bytes of features per head.
+struct DirectExtra64 {
+  int src_off, row_bytes;
+  __device__ __forceinline__ static int source(int row_bytes, int wave, int lane, int rows_left) {
+    const int row = 4 * wave + (lane >> 4);
+    const int piece = (lane & 15) ^ tile_swizzle(row);
+    int key = row + 32 * (piece >> 3);
+    key = key < rows_left ? key : rows_left - 1;
+    return key * row_bytes + 256 + ((piece & 7) << 4);
+  }
+  __device__ __forceinline__ void init(int row_bytes_, int wave, int lane) {
+    row_bytes = row_bytes_;
+    src_off = source(row_bytes_, wave, lane, 64);
+  }
+  __device__ __forceinline__ void issue(const char* tile_src, int rows_left, char* slot, int wave, int lane) const {
+    if (rows_left >= 64) load_lds16(tile_src, src_off, slot + wave * 1024);
+    else load_lds16(tile_src, source(row_bytes, wave, lane, rows_left), slot + wave * 1024);
+  }
+};
+
 // Per-lane offsets for reading a packed swizzled tile.
 // straight_offset(c, piece): fragment of row c (+ a multiple of 16 rows added by the caller as
 // rows * 256 bytes), features 8*piece .. 8*piece+7.

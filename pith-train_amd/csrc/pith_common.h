@@ -20,6 +20,9 @@ int check_launch(const char* what);
 // Compute units of the current device (looked up once per device; 0 if the runtime cannot tell).
 int compute_units();
 
+// Work split of the query-stationary direct-load kernels (forward, dQ): true = 128-row workgroups.
+bool prefer_half_rows(int64_t Sq, int64_t Hq, int64_t B, bool causal);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;

@@ -105,7 +105,14 @@ int pith_combine(const pith_combine_args* args, pith_stream_t stream);
  * LSE_e = LSE_2 * ln 2).
  * q [B,Sq,Hq,Dqk], k [B,Skv,Hkv,Dqk], v [B,Skv,Hkv,Dv], o [B,Sq,Hq,Dv] bf16; lse [B,Hq,Sq] fp32.
  * Query head h reads kv head h / (Hq/Hkv). causal != 0 masks key j > query i and needs
- * Sq == Skv. Supported (Dqk, Dv): (64,64), (128,128), (192,128). Sq and Skv are arbitrary. */
+ * Sq == Skv. Supported (Dqk, Dv): (64,64), (128,128), (192,128). Sq and Skv are arbitrary.
+ *
+ * Keys in two parts (k_pe != NULL; MLA, Dqk = 192, Dv = 128 only): the layer's key is
+ * [k_nope (128 features, per head) | k_pe (64 rotary features, ONE vector per position shared by
+ * all heads)], pithtrain/models/deepseek_v2_lite.py:448-454, where the reference materialises it
+ * with k_pe broadcast to every head. Here k is then k_nope [B,Skv,Hkv,128] and k_pe [B,Skv,64]
+ * (batch stride k_pe_bs, row stride k_pe_rs, elements: it may be a column slice of a wider
+ * tensor) is read beside it; results equal those of the assembled key. */
 typedef struct {
   const void* q;
   const void* k;
@@ -117,6 +124,8 @@ typedef struct {
   int64_t lse_bs, lse_hs;
   float scale;
   int32_t causal;
+  const void* k_pe;          /* NULL: k holds all Dqk features */
+  int64_t k_pe_bs, k_pe_rs;  /* batch / row strides of k_pe, elements */
 } pith_attn_fwd_args;
 
 int pith_attn_fwd(const pith_attn_fwd_args* args, pith_stream_t stream);
@@ -148,7 +157,13 @@ int pith_attn_bwd_delta(const pith_attn_delta_args* args, pith_stream_t stream);
  * accumulate_dq != 0 adds to the existing contents of dq instead of overwriting (the ring's
  * `dq += dq_s`, ring_attention/mla.py:116, done in the kernel epilogue); the same for
  * accumulate_dkv. With Hq > Hkv, dk/dv of a kv head sum over its Hq/Hkv query heads.
- * pith_attn_bwd_dkdv ignores dq; pith_attn_bwd_dq ignores dk, dv. */
+ * pith_attn_bwd_dkdv ignores dq; pith_attn_bwd_dq ignores dk, dv.
+ *
+ * Keys in two parts (k_pe != NULL, see pith_attn_fwd_args; needs Hq == Hkv): k and dk are
+ * [B,Skv,Hkv,128] (the nope part and its gradient); dk_pe [B,Skv,64] (batch stride dk_pe_bs,
+ * contiguous rows, dkv_dtype) receives the gradient of the shared rotary part, i.e. the sum over
+ * heads of the last 64 features of the assembled key's gradient, added in head order through the
+ * workspace (required then: pith_attn_bwd_dkdv_workspace_bytes). */
 typedef struct {
   const void* q;
   const void* k;
@@ -169,6 +184,10 @@ typedef struct {
   int32_t accumulate_dq, accumulate_dkv;
   void* workspace;         /* optional device scratch for pith_attn_bwd_dkdv, 16-byte aligned; may be NULL */
   int64_t workspace_bytes; /* its size */
+  const void* k_pe;          /* NULL: k holds all Dqk features */
+  int64_t k_pe_bs, k_pe_rs;  /* batch / row strides of k_pe, elements */
+  void* dk_pe;               /* pith_attn_bwd_dkdv with k_pe: gradient of k_pe */
+  int64_t dk_pe_bs;
 } pith_attn_bwd_args;
 
 int pith_attn_bwd_dkdv(const pith_attn_bwd_args* args, pith_stream_t stream);

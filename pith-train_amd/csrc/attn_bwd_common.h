@@ -23,6 +23,12 @@ struct BwdParams {
   int split;        // dK/dV kernel: query-head groups are cut into `split` parts handled by different workgroups
   float* ws_dk;     // dK/dV kernel, split > 1: fp32 partial results [split][B][Skv][Hkv][D]
   float* ws_dv;
+  // keys in two parts (k_pe != nullptr): k / dk hold the first 128 features per head; k_pe holds the
+  // last 64, one vector per position shared by all heads (batch / row strides in elements);
+  // ws_dkpe: dK/dV kernel, fp32 per-head gradients of k_pe [Hkv][B][Skv][64]
+  const __bf16* k_pe;
+  int64_t k_pe_bs, k_pe_rs;
+  float* ws_dkpe;
 };
 
 // Stores 4 consecutive output features held by one lane; OutT is __bf16 or float.

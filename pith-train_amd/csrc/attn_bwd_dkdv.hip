@@ -171,7 +171,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
 
   const int64_t q_row_stride = (int64_t)p.Hq * DQK;
   const int64_t do_row_stride = (int64_t)p.Hq * DV;
-  const int64_t k_row_stride = (int64_t)p.Hkv * DQK;
+  // keys in two parts (192-feature keys only): k and dk rows hold 128 features per head, the last 64
+  // features come from k_pe (one vector per position) and their gradient goes, per head, to ws_dkpe
+  const bool two_part = DQK == 192 && p.k_pe != nullptr;
+  const int k_head = two_part ? 128 : DQK;
+  const int64_t k_row_stride = (int64_t)p.Hkv * k_head;
   const int64_t v_row_stride = (int64_t)p.Hkv * DV;
 
   // stationary fragments: K rows for wave A, V rows for wave B
@@ -179,9 +183,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
   {
     const int row = key < p.Skv ? key : p.Skv - 1;
     if (!role_b) {
-      const __bf16* src = p.k + b * p.k_bs + row * k_row_stride + (int64_t)hk * DQK + g * 8;
+      const __bf16* src = p.k + b * p.k_bs + row * k_row_stride + (int64_t)hk * k_head + g * 8;
+      const __bf16* src_pe = two_part ? p.k_pe + b * p.k_pe_bs + row * p.k_pe_rs + g * 8 : src + 128;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) stat[ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
+      for (int ks = 0; ks < KS; ++ks)
+        stat[ks] = *reinterpret_cast<const bf16x8*>(ks < 8 ? src + ks * 16 : src_pe + (ks - 8) * 16);
     } else {
       const __bf16* src = p.v + b * p.v_bs + row * v_row_stride + (int64_t)hk * DV + g * 8;
 #pragma unroll
@@ -241,9 +247,19 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
 
   // ---- epilogue: wave A stores dV, wave B stores dK, for key row `key`, features 32*o + 8*b4 + 4*g ..+3
   if (key < p.Skv) {
-    const int d = role_b ? DQK : DV;
-    const int nblk = role_b ? DB : DVB;
+    const int d = role_b ? k_head : DV;
+    const int nblk = role_b ? k_head / 32 : DVB;
     const int64_t row_stride = role_b ? k_row_stride : v_row_stride;
+    if (two_part && role_b) {  // this head's gradient of the shared rotary part: [Hkv][B][Skv][64] fp32
+      float* ws = p.ws_dkpe + (((int64_t)hk * p.B + b) * p.Skv + key) * 64;
+#pragma unroll
+      for (int o = 4; o < NACC; ++o)
+        if (o < DB)
+#pragma unroll
+          for (int b4 = 0; b4 < 4; ++b4)
+            store4<float>(ws + 32 * (o - 4) + 8 * b4 + 4 * g, acc[o][4 * b4], acc[o][4 * b4 + 1], acc[o][4 * b4 + 2],
+                          acc[o][4 * b4 + 3], false);
+    }
     if (p.split > 1) {
       float* ws = (role_b ? p.ws_dk : p.ws_dv) +
                   (((int64_t)part * p.B + b) * p.Skv + key) * row_stride + (int64_t)hk * d;
@@ -303,10 +319,16 @@ int pick_split(const pith_attn_bwd_args* a) {
   return split;
 }
 
-int64_t workspace_bytes_for(const pith_attn_bwd_args* a, int split) {
+// Workspace layout: [head-split partial dK | partial dV] (split > 1), then the per-head gradients of a
+// shared k_pe [Hkv][B][Skv][64] (keys in two parts).
+int64_t split_bytes_for(const pith_attn_bwd_args* a, int split) {
   if (split <= 1) return 0;
   return (int64_t)split * a->B * a->Skv * a->Hkv * (a->Dqk + a->Dv) * (int64_t)sizeof(float);
 }
+int64_t dkpe_bytes_for(const pith_attn_bwd_args* a) {
+  return a->k_pe ? a->Hkv * a->B * a->Skv * 64 * (int64_t)sizeof(float) : 0;
+}
+int64_t workspace_bytes_for(const pith_attn_bwd_args* a, int split) { return split_bytes_for(a, split) + dkpe_bytes_for(a); }
 
 template <int DQK, int DV>
 void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
@@ -324,6 +346,25 @@ void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
       if (f32) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, false, float>), grid, block, 0, st, p);
       else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, false, __bf16>), grid, block, 0, st, p);
     }
+  }
+  if (p.k_pe) {  // dk_pe (+)= sum over heads, in head order
+    ReduceParams r;
+    r.row_elems[0] = 64;
+    r.part_stride[0] = a->B * a->Skv * 64;
+    r.n4[0] = r.part_stride[0] / 4;
+    r.ws[0] = p.ws_dkpe;
+    r.out[0] = a->dk_pe;
+    r.out_bs[0] = a->dk_pe_bs;
+    r.row_elems[1] = r.part_stride[1] = r.n4[1] = r.out_bs[1] = 0;
+    r.ws[1] = nullptr;
+    r.out[1] = nullptr;
+    r.rows_per_batch = a->Skv;
+    r.parts = (int)a->Hkv;
+    r.accumulate = a->accumulate_dkv;
+    const int64_t blocks = (r.n4[0] + 255) / 256;
+    const dim3 rgrid((unsigned)(blocks < 8192 ? blocks : 8192), 1);
+    if (f32) hipLaunchKernelGGL((reduce_parts_kernel<float>), rgrid, dim3(256), 0, st, r);
+    else hipLaunchKernelGGL((reduce_parts_kernel<__bf16>), rgrid, dim3(256), 0, st, r);
   }
   if (p.split > 1) {
     ReduceParams r;
@@ -366,6 +407,14 @@ int run_dkdv(const pith_attn_bwd_args* a, int split, void* workspace, hipStream_
     return fail(PITH_ERR_UNSUPPORTED, "%s: Skv=%lld x Hkv=%lld x B=%lld exceeds the launch grid limit", who,
                 (long long)a->Skv, (long long)a->Hkv, (long long)a->B);
   BwdParams p = make_bwd_params(a);
+  if (a->k_pe) {
+    if (a->Hq != a->Hkv)
+      return fail(PITH_ERR_UNSUPPORTED, "%s: keys in two parts need Hq == Hkv (got %lld, %lld)", who, (long long)a->Hq, (long long)a->Hkv);
+    if (!a->dk_pe) return fail(PITH_ERR_NULL_POINTER, "%s: dk_pe is NULL", who);
+    if (!aligned16(a->dk_pe) || a->dk_pe_bs % 8) return fail(PITH_ERR_MISALIGNED, "%s: dk_pe pointer / batch stride must keep 16-byte alignment", who);
+    if (!workspace) return fail(PITH_ERR_BAD_SHAPE, "%s: keys in two parts need a workspace of %lld bytes", who, (long long)dkpe_bytes_for(a));
+    p.ws_dkpe = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + split_bytes_for(a, split));
+  }
   begin_launch();
   if (split > 1 && workspace) {
     p.split = split;
@@ -413,12 +462,11 @@ extern "C" int pith_attn_bwd_dkdv(const pith_attn_bwd_args* a, pith_stream_t str
   if (rc != PITH_OK) return rc;
   // Head groups are split only when the caller brought a workspace that is large enough.
   int split = pick_split(a);
-  const int64_t need = workspace_bytes_for(a, split);
-  if (split > 1 && a->workspace && a->workspace_bytes >= need) {
-    if (!aligned16(a->workspace)) return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_dkdv: workspace must be 16-byte aligned");
-  } else {
-    split = 1;
-  }
+  if (!(split > 1 && a->workspace && a->workspace_bytes >= workspace_bytes_for(a, split))) split = 1;
+  if (a->workspace && !aligned16(a->workspace)) return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_dkdv: workspace must be 16-byte aligned");
+  if (a->k_pe && (!a->workspace || a->workspace_bytes < workspace_bytes_for(a, split)))
+    return fail(PITH_ERR_BAD_SHAPE, "pith_attn_bwd_dkdv: keys in two parts need a workspace of %lld bytes, %lld given",
+                (long long)workspace_bytes_for(a, split), (long long)(a->workspace ? a->workspace_bytes : 0));
   return run_dkdv(a, split, a->workspace, (hipStream_t)stream, "pith_attn_bwd_dkdv");
 }
 

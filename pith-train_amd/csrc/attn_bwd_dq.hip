@@ -260,6 +260,13 @@ int validate_bwd(const pith_attn_bwd_args* a, const char* who, bool need_dq, boo
     return fail(PITH_ERR_MISALIGNED, "%s: dq pointer / batch stride must keep 16-byte alignment", who);
   if (need_dkv && (!aligned16(a->dk) || !aligned16(a->dv) || a->dk_bs % 8 || a->dv_bs % 8))
     return fail(PITH_ERR_MISALIGNED, "%s: dk/dv pointers / batch strides must keep 16-byte alignment", who);
+  if (a->k_pe) {
+    if (a->Dqk != 192 || a->Dv != 128)
+      return fail(PITH_ERR_UNSUPPORTED, "%s: keys in two parts (k_pe) need head dims (192, 128), got (%lld, %lld)", who,
+                  (long long)a->Dqk, (long long)a->Dv);
+    if (!aligned16(a->k_pe) || a->k_pe_bs % 8 || a->k_pe_rs % 8 || a->k_pe_rs < 64)
+      return fail(PITH_ERR_MISALIGNED, "%s: k_pe pointer / strides must keep 16-byte alignment (row stride >= 64)", who);
+  }
   const bool dims_ok = (a->Dqk == 128 && a->Dv == 128) || (a->Dqk == 192 && a->Dv == 128) || (a->Dqk == 64 && a->Dv == 64);
   if (!dims_ok)
     return fail(PITH_ERR_UNSUPPORTED, "%s: head dims (Dqk=%lld, Dv=%lld) not in {(64,64),(128,128),(192,128)}", who,
@@ -281,6 +288,8 @@ BwdParams make_bwd_params(const pith_attn_bwd_args* a) {
   p.split = 1;
   p.ws_dk = nullptr;
   p.ws_dv = nullptr;
+  p.k_pe = (const __bf16*)a->k_pe; p.k_pe_bs = a->k_pe_bs; p.k_pe_rs = a->k_pe_rs;
+  p.ws_dkpe = nullptr;
   return p;
 }
 

@@ -73,8 +73,13 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
 
   const int64_t q_row_stride = (int64_t)p.Hq * DQK;
   const int64_t do_row_stride = (int64_t)p.Hq * kDv;
-  const int k_row_bytes = p.Hkv * DQK * 2, v_row_bytes = p.Hkv * kDv * 2;
-  const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * DQK);
+  // keys in two parts: K rows hold 128 features per head, the last 64 come from k_pe (no head offset)
+  const bool two_part = DQK == 192 && p.k_pe != nullptr;
+  const int k_head_elems = two_part ? 128 : DQK;
+  const int k_row_bytes = p.Hkv * k_head_elems * 2, v_row_bytes = p.Hkv * kDv * 2;
+  const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * k_head_elems);
+  const char* kx = two_part ? reinterpret_cast<const char*>(p.k_pe + b * p.k_pe_bs) : kh;  // source of features 128..
+  const int kx_row_bytes = two_part ? (int)p.k_pe_rs * 2 : k_row_bytes;
   const char* vh = reinterpret_cast<const char*>(p.v + b * p.v_bs + (int64_t)hk * kDv);
 
   const int n_tiles_all = (p.Skv + kBN - 1) / kBN;
@@ -89,14 +94,14 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   mover.init(v_row_bytes, wave, lane);
   if constexpr (DQK != kDv) {
     kmover.init(k_row_bytes, wave, lane);
-    xmover.init(k_row_bytes, wave, lane);
+    xmover.init(kx_row_bytes, two_part ? 0 : 256, wave, lane);
   }
   auto request = [&](int t) __attribute__((always_inline)) {
     char* kslot = kbuf + (t & (kSlots - 1)) * kKTile;
     const char* ksrc = kh + (int64_t)t * kBN * k_row_bytes;
     if constexpr (DQK != kDv) {
       kmover.issue(ksrc, p.Skv - t * kBN, kslot, wave, lane);
-      xmover.issue(ksrc, p.Skv - t * kBN, kslot + kTile, wave, lane);
+      xmover.issue(kx + (int64_t)t * kBN * kx_row_bytes, p.Skv - t * kBN, kslot + kTile, wave, lane);
     } else {
       mover.issue(ksrc, p.Skv - t * kBN, kslot, wave, lane);
     }

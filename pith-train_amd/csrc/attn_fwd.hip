@@ -283,6 +283,14 @@ extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) 
   p.B = (int)a->B; p.m_tiles = 0;
   p.q_bs = a->q_bs; p.k_bs = a->k_bs; p.v_bs = a->v_bs; p.o_bs = a->o_bs; p.lse_bs = a->lse_bs; p.lse_hs = a->lse_hs;
   p.kappa = a->scale * 1.44269504088896340736f;
+  p.k_pe = (const __bf16*)a->k_pe; p.k_pe_bs = a->k_pe_bs; p.k_pe_rs = a->k_pe_rs;
+  if (a->k_pe) {
+    if (a->Dqk != 192 || a->Dv != 128)
+      return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: keys in two parts (k_pe) need head dims (192, 128), got (%lld, %lld)",
+                  (long long)a->Dqk, (long long)a->Dv);
+    if (!aligned16(a->k_pe) || a->k_pe_bs % 8 || a->k_pe_rs % 8 || a->k_pe_rs < 64)
+      return fail(PITH_ERR_MISALIGNED, "pith_attn_fwd: k_pe pointer / strides must keep 16-byte alignment (row stride >= 64)");
+  }
   hipStream_t st = (hipStream_t)stream;
   begin_launch();
   if ((a->Dqk == 128 || a->Dqk == 192) && a->Dv == 128) {

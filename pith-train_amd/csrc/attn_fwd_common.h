@@ -18,6 +18,10 @@ struct FwdParams {
   int B, m_tiles;
   int64_t q_bs, k_bs, v_bs, o_bs, lse_bs, lse_hs;
   float kappa;  // scale * log2(e)
+  // keys in two parts (k_pe != nullptr): k holds the first 128 features per head, k_pe the last 64,
+  // one vector per position shared by all heads (batch / row strides in elements)
+  const __bf16* k_pe;
+  int64_t k_pe_bs, k_pe_rs;
 };
 
 // Forward for head dims (128, 128) and (192, 128) with tiles loaded global -> LDS directly:

@@ -72,9 +72,14 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
 
   const int64_t q_row_stride = (int64_t)p.Hq * DQK;
   const int64_t o_row_stride = (int64_t)p.Hq * kDv;
-  const int k_row_bytes = p.Hkv * DQK * 2, v_row_bytes = p.Hkv * kDv * 2;
+  // keys in two parts: K rows hold 128 features per head, the last 64 come from k_pe (no head offset)
+  const bool two_part = DQK == 192 && p.k_pe != nullptr;
+  const int k_head_elems = two_part ? 128 : DQK;
+  const int k_row_bytes = p.Hkv * k_head_elems * 2, v_row_bytes = p.Hkv * kDv * 2;
   const __bf16* qh = p.q + b * p.q_bs + (int64_t)h * DQK;
-  const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * DQK);
+  const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * k_head_elems);
+  const char* kx = two_part ? reinterpret_cast<const char*>(p.k_pe + b * p.k_pe_bs) : kh;  // source of features 128..
+  const int kx_row_bytes = two_part ? (int)p.k_pe_rs * 2 : k_row_bytes;
   const char* vh = reinterpret_cast<const char*>(p.v + b * p.v_bs + (int64_t)hk * kDv);
 
   // Number of key tiles this workgroup / this wavefront has to visit.
@@ -90,14 +95,14 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   mover.init(v_row_bytes, wave, lane);
   if constexpr (DQK != kDv) {
     kmover.init(k_row_bytes, wave, lane);
-    xmover.init(k_row_bytes, wave, lane);
+    xmover.init(kx_row_bytes, two_part ? 0 : 256, wave, lane);
   }
   auto issue_k = [&](int t) __attribute__((always_inline)) {
     char* slot = kbuf + (t & (kSlots - 1)) * kKTile;
     const char* src = kh + (int64_t)t * kBN * k_row_bytes;
     if constexpr (DQK != kDv) {
       kmover.issue(src, p.Skv - t * kBN, slot, wave, lane);
-      xmover.issue(src, p.Skv - t * kBN, slot + kTile, wave, lane);
+      xmover.issue(kx + (int64_t)t * kBN * kx_row_bytes, p.Skv - t * kBN, slot + kTile, wave, lane);
     } else {
       mover.issue(src, p.Skv - t * kBN, slot, wave, lane);
     }

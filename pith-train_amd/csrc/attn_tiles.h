@@ -234,21 +234,25 @@ constexpr int kExtraTileBytes = 32 * kRowBytes128;
 // Moves that part of a tile global memory -> LDS: one global_load_lds per thread of a 512-thread
 // workgroup (wave w fills LDS rows 4w .. 4w+3). Source rows are 384 bytes of features per head.
 struct DirectExtra64 {
-  int src_off, row_bytes;
-  __device__ __forceinline__ static int source(int row_bytes, int wave, int lane, int rows_left) {
+  int src_off, row_bytes, col_bytes;
+  __device__ __forceinline__ static int source(int row_bytes, int col_bytes, int wave, int lane, int rows_left) {
     const int row = 4 * wave + (lane >> 4);
     const int piece = (lane & 15) ^ tile_swizzle(row);
     int key = row + 32 * (piece >> 3);
     key = key < rows_left ? key : rows_left - 1;
-    return key * row_bytes + 256 + ((piece & 7) << 4);
+    return key * row_bytes + col_bytes + ((piece & 7) << 4);
   }
-  __device__ __forceinline__ void init(int row_bytes_, int wave, int lane) {
+  // row_bytes: distance between consecutive source rows; col_bytes: where the 64 features start
+  // within a source row (256 when they follow the first 128 features of the same row, 0 when they
+  // are a tensor of their own)
+  __device__ __forceinline__ void init(int row_bytes_, int col_bytes_, int wave, int lane) {
     row_bytes = row_bytes_;
-    src_off = source(row_bytes_, wave, lane, 64);
+    col_bytes = col_bytes_;
+    src_off = source(row_bytes_, col_bytes_, wave, lane, 64);
   }
   __device__ __forceinline__ void issue(const char* tile_src, int rows_left, char* slot, int wave, int lane) const {
     if (rows_left >= 64) load_lds16(tile_src, src_off, slot + wave * 1024);
-    else load_lds16(tile_src, source(row_bytes, wave, lane, rows_left), slot + wave * 1024);
+    else load_lds16(tile_src, source(row_bytes, col_bytes, wave, lane, rows_left), slot + wave * 1024);
   }
 };
 

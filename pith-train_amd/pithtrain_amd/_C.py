@@ -54,6 +54,7 @@ class AttnFwdArgs(Structure):
         ("q_bs", c_int64), ("k_bs", c_int64), ("v_bs", c_int64), ("o_bs", c_int64),
         ("lse_bs", c_int64), ("lse_hs", c_int64),
         ("scale", c_float), ("causal", c_int32),
+        ("k_pe", c_void_p), ("k_pe_bs", c_int64), ("k_pe_rs", c_int64),
     ]  # fmt: skip
 
 
@@ -78,6 +79,8 @@ class AttnBwdArgs(Structure):
         ("dq_dtype", c_int32), ("dkv_dtype", c_int32),
         ("accumulate_dq", c_int32), ("accumulate_dkv", c_int32),
         ("workspace", c_void_p), ("workspace_bytes", c_int64),
+        ("k_pe", c_void_p), ("k_pe_bs", c_int64), ("k_pe_rs", c_int64),
+        ("dk_pe", c_void_p), ("dk_pe_bs", c_int64),
     ]  # fmt: skip
 
 

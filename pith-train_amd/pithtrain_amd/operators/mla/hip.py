@@ -27,7 +27,23 @@ from pithtrain_amd import _C
 SUPPORTED_HEAD_DIMS = ((64, 64), (128, 128), (192, 128))
 
 
-def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool) -> None:
+def _k_pe_strides(k: torch.Tensor, k_pe: torch.Tensor):
+    """Checks the shared rotary key part k_pe ([b, s, 64] or [b, s, 1, 64], unit stride along the
+    features; it may be a column slice of a wider tensor) against k_nope and returns
+    (tensor viewed as [b, s, 64], batch stride, row stride) in elements."""
+    if k_pe.dim() == 4:
+        assert k_pe.shape[2] == 1, "k_pe must have a single head"
+        k_pe = k_pe[:, :, 0]
+    b, s = k.shape[0], k.shape[1]
+    assert k_pe.dtype == torch.bfloat16 and tuple(k_pe.shape) == (b, s, 64), (
+        f"k_pe of shape {tuple(k_pe.shape)} does not match [b={b}, s={s}, 64]"
+    )
+    assert k_pe.stride(2) == 1, "k_pe is not contiguous along its last dim"
+    rs = k_pe.stride(1) if s > 1 else 64
+    return k_pe, (k_pe.stride(0) if b > 1 else s * rs), rs
+
+
+def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool, k_pe=None) -> None:
     _C.require_device(q, k, v)
     assert q.dtype == k.dtype == v.dtype == torch.bfloat16, "q, k, v must be bfloat16"
     assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be [B, S, H, D]"
@@ -35,7 +51,14 @@ def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool) 
     assert (d_q, d_v) in SUPPORTED_HEAD_DIMS, (
         f"HIP attention kernels support (dq, dv) in {SUPPORTED_HEAD_DIMS}, got dq={d_q} and dv={d_v}"
     )
-    assert k.shape[-1] == d_q, f"k head dim {k.shape[-1]} != q head dim {d_q}"
+    if k_pe is not None:
+        _C.require_device(q, k_pe)
+        assert (d_q, d_v) == (192, 128) and k.shape[-1] == 128, (
+            "keys in two parts (k_nope, k_pe) need dq=192, dv=128 and a 128-feature k_nope"
+        )
+        assert q.shape[2] == k.shape[2], "keys in two parts need as many kv heads as query heads"
+    else:
+        assert k.shape[-1] == d_q, f"k head dim {k.shape[-1]} != q head dim {d_q}"
     assert k.shape[0] == q.shape[0] and v.shape[0] == q.shape[0], "batch sizes differ"
     assert k.shape[1] == v.shape[1] and k.shape[2] == v.shape[2], "k and v disagree on sequence length or heads"
     assert q.shape[2] % k.shape[2] == 0, f"q heads {q.shape[2]} not a multiple of kv heads {k.shape[2]}"
@@ -45,10 +68,14 @@ def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool) 
 
 def attn_fwd_into(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
-    softmax_scale: float, causal: bool,
+    softmax_scale: float, causal: bool, k_pe: torch.Tensor = None,
 ) -> None:  # fmt: skip
-    """o, lse <- attention(q, k, v). o [b, sq, hq, dv] bf16 and lse [b, hq, sq] fp32 are written."""
-    _check_qkv(q, k, v, causal)
+    """o, lse <- attention(q, k, v). o [b, sq, hq, dv] bf16 and lse [b, hq, sq] fp32 are written.
+
+    With k_pe ([b, skv, 64], the MLA layer's rotary key part, one vector per position shared by all
+    heads) k is the 128-feature k_nope and the key of head h is [k[:, :, h] | k_pe]: what
+    pithtrain/models/deepseek_v2_lite.py:448-454 materialises is read in place instead."""
+    _check_qkv(q, k, v, causal, k_pe)
     _C.require_device(q, o, lse)
     b, sq, hq, d_q = q.shape
     _, skv, hkv, d_v = v.shape
@@ -61,7 +88,11 @@ def attn_fwd_into(
         q_bs=_C.bshd_batch_stride(q, "q"), k_bs=_C.bshd_batch_stride(k, "k"),
         v_bs=_C.bshd_batch_stride(v, "v"), o_bs=_C.bshd_batch_stride(o, "o"),
         lse_bs=lse_bs, lse_hs=lse_hs, scale=float(softmax_scale), causal=int(bool(causal)),
+        k_pe=None, k_pe_bs=0, k_pe_rs=0,
     )  # fmt: skip
+    if k_pe is not None:
+        k_pe, args.k_pe_bs, args.k_pe_rs = _k_pe_strides(k, k_pe)
+        args.k_pe = k_pe.data_ptr()
     _C.check(_C.lib().pith_attn_fwd(_C.byref(args), _C.current_stream(q)))
 
 
@@ -80,8 +111,8 @@ def attn_bwd_delta_into(out: torch.Tensor, dout: torch.Tensor, delta: torch.Tens
     _C.check(_C.lib().pith_attn_bwd_delta(_C.byref(args), _C.current_stream(out)))
 
 
-def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal) -> _C.AttnBwdArgs:
-    _check_qkv(q, k, v, causal)
+def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe=None) -> _C.AttnBwdArgs:
+    _check_qkv(q, k, v, causal, k_pe)
     _C.require_device(q, dout, lse, delta)
     b, sq, hq, d_q = q.shape
     _, skv, hkv, d_v = v.shape
@@ -90,7 +121,12 @@ def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal) -> _C.AttnBwdArg
         assert t.dtype == torch.float32 and tuple(t.shape) == (b, hq, sq), f"{name} has the wrong dtype or shape"
     lse_bs, lse_hs = _C.bhs_strides(lse, "lse")
     assert _C.bhs_strides(delta, "delta") == (lse_bs, lse_hs), "lse and delta must share strides"
+    kpe_ptr, kpe_bs, kpe_rs = None, 0, 0
+    if k_pe is not None:
+        k_pe, kpe_bs, kpe_rs = _k_pe_strides(k, k_pe)
+        kpe_ptr = k_pe.data_ptr()
     return _C.AttnBwdArgs(
+        k_pe=kpe_ptr, k_pe_bs=kpe_bs, k_pe_rs=kpe_rs, dk_pe=None, dk_pe_bs=0,
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), dout=dout.data_ptr(),
         lse=lse.data_ptr(), delta=delta.data_ptr(), dq=None, dk=None, dv=None,
         B=b, Sq=sq, Skv=skv, Hq=hq, Hkv=hkv, Dqk=d_q, Dv=d_v,
@@ -105,12 +141,22 @@ def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal) -> _C.AttnBwdArg
 
 def attn_bwd_dkdv_into(
     q, k, v, dout, lse, delta, dk: torch.Tensor, dv: torch.Tensor, softmax_scale: float, causal: bool,
-    accumulate: bool = False,
+    accumulate: bool = False, k_pe: torch.Tensor = None, dk_pe: torch.Tensor = None,
 ) -> None:  # fmt: skip
-    """dk, dv <- (or +=, with accumulate) the gradients of this chunk pair; bf16 or fp32 outputs."""
-    args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal)
+    """dk, dv <- (or +=, with accumulate) the gradients of this chunk pair; bf16 or fp32 outputs.
+    With k_pe (see attn_fwd_into) dk is the gradient of k_nope and dk_pe [b, skv, 64] (contiguous rows,
+    same dtype as dk) receives the gradient of k_pe, summed over heads in head order."""
+    args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe)
     _C.require_device(q, dk, dv)
     assert dk.shape == k.shape and dv.shape == v.shape and dk.dtype == dv.dtype, "dk/dv must match k/v"
+    if k_pe is not None:
+        assert dk_pe is not None, "keys in two parts need a dk_pe tensor"
+        _C.require_device(q, dk_pe)
+        b, s = k.shape[0], k.shape[1]
+        assert tuple(dk_pe.shape) == (b, s, 64) and dk_pe.dtype == dk.dtype, "dk_pe must be [b, skv, 64] in dk's dtype"
+        assert dk_pe.stride(2) == 1 and (s == 1 or dk_pe.stride(1) == 64), "dk_pe rows are not contiguous"
+        args.dk_pe = dk_pe.data_ptr()
+        args.dk_pe_bs = dk_pe.stride(0) if b > 1 else s * 64
     args.dk, args.dv = dk.data_ptr(), dv.data_ptr()
     args.dk_bs, args.dv_bs = _C.bshd_batch_stride(dk, "dk"), _C.bshd_batch_stride(dv, "dv")
     args.dkv_dtype = _C.dtype_code(dk)
@@ -127,9 +173,10 @@ def attn_bwd_dkdv_into(
 
 def attn_bwd_dq_into(
     q, k, v, dout, lse, delta, dq: torch.Tensor, softmax_scale: float, causal: bool, accumulate: bool = False,
+    k_pe: torch.Tensor = None,
 ) -> None:  # fmt: skip
     """dq <- (or +=, with accumulate) the query gradient of this chunk pair; bf16 or fp32 output."""
-    args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal)
+    args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe)
     _C.require_device(q, dq)
     assert dq.shape == q.shape, "dq must match q"
     args.dq = dq.data_ptr()
@@ -143,12 +190,14 @@ def attn_bwd_dq_into(
 # Reference-named helpers (pithtrain/operators/mla/triton.py:552-603)
 
 
-def _mla_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float, causal: bool = True):
-    """Raw attention forward. Returns (out, lse) with lse in log2 scale."""
+def _mla_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float, causal: bool = True,
+             *, k_pe: torch.Tensor = None):  # fmt: skip
+    """Raw attention forward. Returns (out, lse) with lse in log2 scale. Keyword k_pe: keys in two
+    parts (k = k_nope), see attn_fwd_into."""
     (b, s, h, _), dv_dim = q.shape, v.shape[-1]
     o = torch.empty((b, s, h, dv_dim), dtype=torch.bfloat16, device=q.device)
     lse = torch.empty((b, h, s), dtype=torch.float32, device=q.device)
-    attn_fwd_into(q, k, v, o, lse, softmax_scale, causal)
+    attn_fwd_into(q, k, v, o, lse, softmax_scale, causal, k_pe)
     return o, lse
 
 
@@ -161,19 +210,26 @@ def _mla_bwd_preprocess(out: torch.Tensor, dout: torch.Tensor):
 
 
 def _mla_bwd_dk_dv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
-                   lse: torch.Tensor, delta: torch.Tensor, softmax_scale: float, causal: bool = True):  # fmt: skip
-    """Phase 2: compute dK and dV using external lse and delta. Returns (dk, dv)."""
+                   lse: torch.Tensor, delta: torch.Tensor, softmax_scale: float, causal: bool = True,
+                   *, k_pe: torch.Tensor = None):  # fmt: skip
+    """Phase 2: compute dK and dV using external lse and delta. Returns (dk, dv), or with keyword k_pe
+    (keys in two parts, k = k_nope) (dk_nope, dv, dk_pe)."""
     dk = torch.empty_like(k)
     dv_out = torch.empty_like(v)
-    attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv_out, softmax_scale, causal)
-    return dk, dv_out
+    if k_pe is None:
+        attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv_out, softmax_scale, causal)
+        return dk, dv_out
+    dk_pe = torch.empty((k.shape[0], k.shape[1], 64), dtype=k.dtype, device=k.device)
+    attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv_out, softmax_scale, causal, k_pe=k_pe, dk_pe=dk_pe)
+    return dk, dv_out, dk_pe
 
 
 def _mla_bwd_dq(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
-                lse: torch.Tensor, delta: torch.Tensor, softmax_scale: float, causal: bool = True):  # fmt: skip
+                lse: torch.Tensor, delta: torch.Tensor, softmax_scale: float, causal: bool = True,
+                *, k_pe: torch.Tensor = None):  # fmt: skip
     """Phase 3: compute dQ using external lse and delta. Returns dq."""
     dq_out = torch.empty_like(q)
-    attn_bwd_dq_into(q, k, v, dout, lse, delta, dq_out, softmax_scale, causal)
+    attn_bwd_dq_into(q, k, v, dout, lse, delta, dq_out, softmax_scale, causal, k_pe=k_pe)
     return dq_out
 
 

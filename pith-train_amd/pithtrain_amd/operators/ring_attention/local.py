@@ -26,6 +26,13 @@ row range writes bf16 directly, which is the same single rounding. dQ is accumul
 in fp32 inside the dQ kernel's epilogue and rounded once (the reference adds bf16 partials,
 mla.py:116). dK/dV of every visited chunk are returned separately, zero where a chunk's rows were
 not visible; on a real ring those are what travels back to the owning ranks (standard.py:164-187).
+
+Keys in two parts (MLA): every function below takes optional `k_pe` chunks ([B, S_l, 64], the
+rotary key part shared by all heads) beside 128-feature `k` chunks (k_nope). The chunk kernels
+then read [k_nope | k_pe] in place of the assembled 192-feature key that the reference builds at
+pithtrain/models/deepseek_v2_lite.py:448-454 (with k_pe broadcast to all heads: 24 MB instead of
+16.5 MB per chunk of 4096 tokens and 16 heads, also on the wire of a real ring), and the
+backward returns dk_nope and the head-summed dk_pe per chunk.
 """
 
 from dataclasses import dataclass
@@ -124,6 +131,11 @@ def _rows(t: torch.Tensor, rows: Tuple[int, int]) -> torch.Tensor:
     return t if rows == (0, t.shape[1]) else t[:, rows[0] : rows[1]]
 
 
+def _pe_rows(t, rows: Tuple[int, int]):
+    """Row range of a [B, S, 64] (or [B, S, 1, 64]) tensor (a view); None passes through."""
+    return t if t is None or rows == (0, t.shape[1]) else t[:, rows[0] : rows[1]]
+
+
 def _lse_rows(t: torch.Tensor, rows: Tuple[int, int]) -> torch.Tensor:
     """Row range of a [B, H, S] tensor (a view)."""
     return t if rows == (0, t.shape[2]) else t[:, :, rows[0] : rows[1]]
@@ -158,7 +170,7 @@ class RingForward:
     def _covers(step: RingStep, r: Tuple[int, int]) -> bool:
         return step.q_rows[0] <= r[0] and r[1] <= step.q_rows[1]
 
-    def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor) -> None:
+    def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor, k_pe_j: torch.Tensor = None) -> None:
         assert st == self.steps[self.done], "ring steps must be fed in schedule order"
         assert k_j.is_contiguous() and v_j.is_contiguous(), "ring attention k or v is not contiguous"
         B, S, H, _ = self.q.shape
@@ -168,13 +180,13 @@ class RingForward:
             # reference's initial state (zeros, finfo.min) returns it unchanged, so it is written
             # straight into the running tensors.
             assert st.causal and st.q_rows == (0, S)
-            attn_fwd_into(self.q, k_j, v_j, self.out, self.lse, self.scale, True)
+            attn_fwd_into(self.q, k_j, v_j, self.out, self.lse, self.scale, True, k_pe_j)
             return
         n_q = st.q_rows[1] - st.q_rows[0]
         so = self.step_out[:, :n_q]
         sl = self.step_lse[: B * H * n_q].view(B, H, n_q)
         attn_fwd_into(_rows(self.q, st.q_rows), _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows), so, sl,
-                      self.scale, False)  # fmt: skip
+                      self.scale, False, _pe_rows(k_pe_j, st.kv_rows))  # fmt: skip
         # Ranges in the same state are merged by one launch.
         groups = {}
         for r in self.ranges:
@@ -211,32 +223,43 @@ class RingBackward:
         self.dq_acc = self.dq if single else torch.empty(q.shape, dtype=torch.float32, device=q.device)
         self.done = 0
 
-    def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor, add_to=None):
-        """Returns (dk_j, dv_j), this rank's contribution to chunk st.kv_rank's gradients.
+    def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor, add_to=None, k_pe_j: torch.Tensor = None):
+        """Returns (dk_j, dv_j), this rank's contribution to chunk st.kv_rank's gradients; with
+        k_pe_j (keys in two parts) (dk_nope_j, dv_j, dk_pe_j).
 
-        With add_to=(dk_acc, dv_acc) (tensors shaped like the chunk, bf16 or fp32) the contribution
-        is ADDED to them inside the kernel epilogue instead, and they are returned: the form a
-        gradient accumulator that travels around the ring with its chunk needs."""
+        With add_to=(dk_acc, dv_acc[, dk_pe_acc]) (tensors shaped like the chunk, bf16 or fp32) the
+        contribution is ADDED to them inside the kernel epilogue instead, and they are returned: the
+        form a gradient accumulator that travels around the ring with its chunk needs."""
         assert st == self.steps[self.done], "ring steps must be fed in schedule order"
+        if k_pe_j is not None and k_pe_j.dim() == 4:
+            k_pe_j = k_pe_j[:, :, 0]
+        dk_pe_j = None
         if add_to is None:
             dk_j, dv_j = torch.empty_like(k_j), torch.empty_like(v_j)
+            outs = [dk_j, dv_j]
+            if k_pe_j is not None:
+                dk_pe_j = torch.empty((k_j.shape[0], k_j.shape[1], k_pe_j.shape[-1]), dtype=k_j.dtype, device=k_j.device)
+                outs.append(dk_pe_j)
             if st.kv_rows != (0, k_j.shape[1]):  # rows of the chunk this rank cannot see get no gradient
-                for t in (dk_j, dv_j):
+                for t in outs:
                     t[:, : st.kv_rows[0]].zero_()
                     t[:, st.kv_rows[1] :].zero_()
         else:
-            dk_j, dv_j = add_to
+            dk_j, dv_j = add_to[0], add_to[1]
+            dk_pe_j = add_to[2] if k_pe_j is not None else None
             assert dk_j.shape == k_j.shape and dv_j.shape == v_j.shape, "accumulators must be shaped like the chunk"
         qs, ds = _rows(self.q, st.q_rows), _rows(self.dout, st.q_rows)
         ks, vs = _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows)
         ls, dl = _lse_rows(self.lse, st.q_rows), _lse_rows(self.delta, st.q_rows)
+        pes = _pe_rows(k_pe_j, st.kv_rows)
         attn_bwd_dkdv_into(qs, ks, vs, ds, ls, dl, _rows(dk_j, st.kv_rows), _rows(dv_j, st.kv_rows),
-                           self.scale, st.causal, accumulate=add_to is not None)  # fmt: skip
+                           self.scale, st.causal, accumulate=add_to is not None, k_pe=pes,
+                           dk_pe=_pe_rows(dk_pe_j, st.kv_rows))  # fmt: skip
         # Step 0 covers every row and initialises the accumulator; later steps add to their rows.
         attn_bwd_dq_into(qs, ks, vs, ds, ls, dl, _rows(self.dq_acc, st.q_rows), self.scale, st.causal,
-                         accumulate=self.done > 0)  # fmt: skip
+                         accumulate=self.done > 0, k_pe=pes)  # fmt: skip
         self.done += 1
-        return dk_j, dv_j
+        return (dk_j, dv_j) if k_pe_j is None else (dk_j, dv_j, dk_pe_j)
 
     def finish(self) -> torch.Tensor:
         assert self.done == len(self.steps), "not every ring step has run"
@@ -248,15 +271,17 @@ class RingBackward:
 def ring_forward_local(
     q: torch.Tensor, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor],
     softmax_scale: float, cp_rank: int, cp_size: int, layout: str = "contiguous",
+    k_pe_chunks: Sequence[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
     """Forward of rank `cp_rank`: returns (out bf16 [B, S_l, Hq, Dv], lse fp32 base-2 [B, Hq, S_l]).
 
     k_chunks[j] / v_chunks[j] are the K/V chunks owned by rank j (entries the schedule never
-    visits may be None)."""
+    visits may be None); with k_pe_chunks the keys come in two parts (k_chunks = k_nope)."""
     steps = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
     fwd = RingForward(q, v_chunks[cp_rank].shape[-1], softmax_scale, steps, layout)
     for st in steps:
-        fwd.run_step(st, k_chunks[st.kv_rank], v_chunks[st.kv_rank])
+        fwd.run_step(st, k_chunks[st.kv_rank], v_chunks[st.kv_rank],
+                     None if k_pe_chunks is None else k_pe_chunks[st.kv_rank])  # fmt: skip
     return fwd.result()
 
 
@@ -264,29 +289,43 @@ def ring_backward_local(
     dout: torch.Tensor, q: torch.Tensor, out: torch.Tensor, lse: torch.Tensor,
     k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor],
     softmax_scale: float, cp_rank: int, cp_size: int, layout: str = "contiguous",
+    k_pe_chunks: Sequence[torch.Tensor] = None,
 ):  # fmt: skip
     """Backward of rank `cp_rank`. Returns (dq, dk_list, dv_list): dq bf16 like q; dk_list[j] and
-    dv_list[j] are this rank's contribution to the gradients of chunk j (None if never visited)."""
+    dv_list[j] are this rank's contribution to the gradients of chunk j (None if never visited).
+    With k_pe_chunks (keys in two parts) a fourth list holds the contributions to every k_pe chunk."""
     steps = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
     bwd = RingBackward(dout, q, out, lse, softmax_scale, steps)
     dk_list: List[torch.Tensor] = [None] * cp_size
     dv_list: List[torch.Tensor] = [None] * cp_size
+    dpe_list: List[torch.Tensor] = [None] * cp_size
     for st in steps:
-        dk_list[st.kv_rank], dv_list[st.kv_rank] = bwd.run_step(st, k_chunks[st.kv_rank], v_chunks[st.kv_rank])
-    return bwd.finish(), dk_list, dv_list
+        j = st.kv_rank
+        if k_pe_chunks is None:
+            dk_list[j], dv_list[j] = bwd.run_step(st, k_chunks[j], v_chunks[j])
+        else:
+            dk_list[j], dv_list[j], dpe_list[j] = bwd.run_step(st, k_chunks[j], v_chunks[j], k_pe_j=k_pe_chunks[j])
+    if k_pe_chunks is None:
+        return bwd.finish(), dk_list, dv_list
+    return bwd.finish(), dk_list, dv_list, dpe_list
 
 
 class RingAttentionLocalFunc(torch.autograd.Function):
-    """autograd wrapper of one rank's ring share; gradients flow to q and to every visited chunk."""
+    """autograd wrapper of one rank's ring share; gradients flow to q and to every visited chunk.
+    *kv holds cp_size K chunks and cp_size V chunks, optionally followed by cp_size k_pe chunks
+    (keys in two parts)."""
 
     @staticmethod
     def forward(ctx, q, softmax_scale, cp_rank, cp_size, layout, *kv):
-        assert len(kv) == 2 * cp_size, "expected cp_size K chunks followed by cp_size V chunks"
-        k_chunks, v_chunks = list(kv[:cp_size]), list(kv[cp_size:])
-        out, lse = ring_forward_local(q, k_chunks, v_chunks, softmax_scale, cp_rank, cp_size, layout)
+        assert len(kv) in (2 * cp_size, 3 * cp_size), "expected cp_size K chunks, cp_size V chunks[, cp_size k_pe chunks]"
+        k_chunks, v_chunks = list(kv[:cp_size]), list(kv[cp_size : 2 * cp_size])
+        pe_chunks = list(kv[2 * cp_size :]) if len(kv) == 3 * cp_size else None
+        out, lse = ring_forward_local(q, k_chunks, v_chunks, softmax_scale, cp_rank, cp_size, layout, pe_chunks)
         visited = sorted({st.kv_rank for st in ring_schedule(cp_rank, cp_size, q.shape[1], layout)})
-        ctx.save_for_backward(q, out, lse, *[k_chunks[j] for j in visited], *[v_chunks[j] for j in visited])
+        kinds = [k_chunks, v_chunks] + ([pe_chunks] if pe_chunks is not None else [])
+        ctx.save_for_backward(q, out, lse, *[kind[j] for kind in kinds for j in visited])
         ctx.visited = visited
+        ctx.n_kinds = len(kinds)
         ctx.conf = (softmax_scale, cp_rank, cp_size, layout)
         return out
 
@@ -296,25 +335,31 @@ class RingAttentionLocalFunc(torch.autograd.Function):
         saved = ctx.saved_tensors
         q, out, lse = saved[0], saved[1], saved[2]
         n = len(ctx.visited)
-        k_chunks, v_chunks = [None] * cp_size, [None] * cp_size
-        for i, j in enumerate(ctx.visited):
-            k_chunks[j], v_chunks[j] = saved[3 + i], saved[3 + n + i]
-        dq, dk_list, dv_list = ring_backward_local(
-            dout, q, out, lse, k_chunks, v_chunks, softmax_scale, cp_rank, cp_size, layout
+        kinds = [[None] * cp_size for _ in range(ctx.n_kinds)]
+        for which in range(ctx.n_kinds):
+            for i, j in enumerate(ctx.visited):
+                kinds[which][j] = saved[3 + which * n + i]
+        grads = ring_backward_local(
+            dout, q, out, lse, kinds[0], kinds[1], softmax_scale, cp_rank, cp_size, layout,
+            kinds[2] if ctx.n_kinds == 3 else None,
         )
-        return (dq, None, None, None, None, *dk_list, *dv_list)
+        return (grads[0], None, None, None, None, *[g for kind in grads[1:] for g in kind])
 
 
 def ring_attention_local(
     q: torch.Tensor, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor],
     softmax_scale: float, cp_rank: int, cp_size: int, layout: str = "contiguous",
+    k_pe_chunks: Sequence[torch.Tensor] = None,
 ) -> torch.Tensor:  # fmt: skip
-    """Differentiable one-GPU ring share for either model family (head dims pick the kernels)."""
+    """Differentiable one-GPU ring share for either model family (head dims pick the kernels).
+    With k_pe_chunks the keys come in two parts (k_chunks = k_nope, see the module docstring)."""
     assert len(k_chunks) == cp_size and len(v_chunks) == cp_size
+    assert k_pe_chunks is None or len(k_pe_chunks) == cp_size
     # Chunks the schedule never visits may be None; autograd needs tensors, so they are replaced
     # by empty placeholders that receive no gradient.
     visited = {st.kv_rank for st in ring_schedule(cp_rank, cp_size, q.shape[1], layout)}
     empty = q.new_empty(0)
     ks = [k_chunks[j] if j in visited else empty for j in range(cp_size)]
     vs = [v_chunks[j] if j in visited else empty for j in range(cp_size)]
-    return RingAttentionLocalFunc.apply(q, softmax_scale, cp_rank, cp_size, layout, *ks, *vs)
+    pes = [] if k_pe_chunks is None else [k_pe_chunks[j] if j in visited else empty for j in range(cp_size)]
+    return RingAttentionLocalFunc.apply(q, softmax_scale, cp_rank, cp_size, layout, *ks, *vs, *pes)

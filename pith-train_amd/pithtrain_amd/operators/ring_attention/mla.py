@@ -40,9 +40,15 @@ def ring_mla_attention_func(
     *,
     layout: str = "contiguous",
     rerotate: bool = False,
+    k_pe: torch.Tensor = None,
 ):
-    """Causal ring MLA attention across context-parallel ranks."""
-    return ring_attention_group_func(q, k, v, softmax_scale, cp_group, layout, rerotate)
+    """Causal ring MLA attention across context-parallel ranks.
+
+    Keyword k_pe: keys in two parts. Pass k = k_nope [B, S_l, H, 128] and k_pe [B, S_l, 64] (or
+    [B, S_l, 1, 64]), the rotary key part that the reference broadcasts to all heads when it assembles
+    key_states (pithtrain/models/deepseek_v2_lite.py:448-454); the kernels read both in place, both
+    rotate around the ring, and autograd returns a gradient for each."""
+    return ring_attention_group_func(q, k, v, softmax_scale, cp_group, layout, rerotate, k_pe)
 
 
 __all__ = ["ring_mla_attention_func", "RingMLAAttentionFunc", "_online_softmax_combine_log2"]

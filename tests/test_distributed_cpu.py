@@ -19,21 +19,27 @@ from oracle import ring_oracle as R
 def _install_cpu_stand_ins():
     from pithtrain_amd.operators.ring_attention import local as L
 
-    def attn_fwd_into(q, k, v, o, lse, scale, causal):
-        ro, rl = R.chunk_fwd(q, k, v, scale, causal)
+    def full_key(k, k_pe):  # keys in two parts: [k_nope | k_pe for every head]
+        return k if k_pe is None else torch.cat([k, k_pe.unsqueeze(2).expand(-1, -1, k.shape[2], -1)], -1)
+
+    def attn_fwd_into(q, k, v, o, lse, scale, causal, k_pe=None):
+        ro, rl = R.chunk_fwd(q, full_key(k, k_pe), v, scale, causal)
         o.copy_(ro)
         lse.copy_(rl)
 
     def attn_bwd_delta_into(out, dout, delta):
         delta.copy_(R.bwd_delta(out, dout))
 
-    def attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, scale, causal, accumulate=False):
-        _, rdk, rdv = R.chunk_bwd(q, k, v, dout, lse.double(), delta.double(), scale, causal)
+    def attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, scale, causal, accumulate=False, k_pe=None, dk_pe=None):
+        _, rdk, rdv = R.chunk_bwd(q, full_key(k, k_pe), v, dout, lse.double(), delta.double(), scale, causal)
+        if k_pe is not None:
+            rpe, rdk = rdk[..., k.shape[-1] :].sum(2), rdk[..., : k.shape[-1]]
+            dk_pe.copy_(dk_pe.double() + rpe if accumulate else rpe)
         dk.copy_(dk.double() + rdk if accumulate else rdk)
         dv.copy_(dv.double() + rdv if accumulate else rdv)
 
-    def attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, scale, causal, accumulate=False):
-        rdq, _, _ = R.chunk_bwd(q, k, v, dout, lse.double(), delta.double(), scale, causal)
+    def attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, scale, causal, accumulate=False, k_pe=None):
+        rdq, _, _ = R.chunk_bwd(q, full_key(k, k_pe), v, dout, lse.double(), delta.double(), scale, causal)
         dq.copy_(dq.double() + rdq if accumulate else rdq)
 
     def combine_into(out1, lse1, out2, lse2, out, lse_out, base=0):
@@ -58,8 +64,8 @@ def _worker(rank, world, port, layout, variant, rerotate, results):
         from pithtrain_amd.operators.ring_attention.standard import ring_attention_func
 
         B, s_l, Hq, Hkv = 1, 16, 4, 2
-        dqk, dv = (24, 16) if variant == "mla" else (16, 16)
-        if variant == "mla":
+        dqk, dv = (24, 16) if variant.startswith("mla") else (16, 16)
+        if variant.startswith("mla"):
             Hkv = Hq
         S = s_l * world
         g = torch.Generator().manual_seed(1234)  # every rank draws the same full sequence
@@ -71,16 +77,27 @@ def _worker(rank, world, port, layout, variant, rerotate, results):
         scale = dqk**-0.5
 
         mine = lambda t: cp_local_slice(t, rank, world, layout).contiguous()  # noqa: E731
-        ql, kl, vl = (mine(t).requires_grad_() for t in (q, k, v))
         group = dist.group.WORLD
-        fn = ring_mla_attention_func if variant == "mla" else ring_attention_func
-        out = fn(ql, kl, vl, scale, group, layout=layout, rerotate=rerotate)
+        if variant == "mla-two-part":
+            # keys in two parts: the last 8 features are one vector per position shared by all heads
+            k_pe = k[:, :, 0, dqk - 8 :].contiguous()
+            k = torch.cat([k[..., : dqk - 8], k_pe.unsqueeze(2).expand(-1, -1, Hkv, -1)], -1).contiguous()
+            ql, kl, vl, pl = (mine(t).requires_grad_() for t in (q, k[..., : dqk - 8], v, k_pe))
+            out = ring_mla_attention_func(ql, kl, vl, scale, group, layout=layout, rerotate=rerotate, k_pe=pl)
+        else:
+            ql, kl, vl = (mine(t).requires_grad_() for t in (q, k, v))
+            fn = ring_mla_attention_func if variant == "mla" else ring_attention_func
+            out = fn(ql, kl, vl, scale, group, layout=layout, rerotate=rerotate)
         out.backward(mine(dout))
 
         ro, rl = R.chunk_fwd(q, k, v, scale, True)
         rdq, rdk, rdv = R.chunk_bwd(q, k, v, dout, rl, R.bwd_delta(ro, dout), scale, True)
         errs = {}
-        for name, got, want in (("O", out, ro), ("dQ", ql.grad, rdq), ("dK", kl.grad, rdk), ("dV", vl.grad, rdv)):
+        checks = [("O", out, ro), ("dQ", ql.grad, rdq), ("dK", kl.grad, rdk), ("dV", vl.grad, rdv)]
+        if variant == "mla-two-part":
+            checks[2] = ("dK nope", kl.grad, rdk[..., : dqk - 8])
+            checks.append(("dK pe", pl.grad, rdk[..., dqk - 8 :].sum(2)))
+        for name, got, want in checks:
             w = mine(want)
             errs[name] = ((got.double() - w).abs().max() / w.abs().max()).item()
         results[rank] = errs
@@ -102,6 +119,8 @@ def _free_port():
         (4, "contiguous", "mla", False), (4, "zigzag", "gqa", False),
         # backward that keeps one K/V chunk per rank and sends the chunks around again
         (2, "zigzag", "gqa", True), (3, "contiguous", "gqa", True), (4, "zigzag", "mla", True),
+        # keys in two parts: k_nope and the shared k_pe both rotate, both receive gradients
+        (3, "zigzag", "mla-two-part", False), (2, "contiguous", "mla-two-part", True),
     ],
 )  # fmt: skip
 def test_ring_over_gloo_matches_full_sequence_attention(world, layout, variant, rerotate):

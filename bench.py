@@ -200,7 +200,7 @@ def bench_ring(torch, args, dev_inputs):
     return ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops
 
 
-def bench_combine(torch, device, reps=50):
+def bench_combine(torch, device, reps=50, graph=True):
     from pithtrain_amd.operators.ring_attention.combine import combine_into
 
     B, S, H, D = 1, 4096, 32, 128
@@ -224,6 +224,8 @@ def bench_combine(torch, device, reps=50):
     for _ in range(8):
         one()
     ms_eager = time_events(torch, one, reps)
+    if not graph:
+        return ms_eager, ms_eager, nbytes, None
     # The same rotating sequence captured once in a HIP graph: a replay enqueues the launches back to
     # back without the host-side cost of each call (the kernel lasts ~25 us, about what the Python
     # binding spends per call), so the time per launch is the kernel's. The library records no memset
@@ -402,7 +404,9 @@ def main():
     ring = bench_ring(torch, args, dev_inputs)
     if ring is None:
         # the HBM-bound kernels, a few dispatches each, for the same counters
-        bench_combine(torch, device, reps=4)
+        del dev_inputs
+        bench_other_config(torch, device, MLA16K, 1, 0)  # the 192/128 kernels, for the same counters
+        bench_combine(torch, device, reps=4, graph=False)
         bench_norm_rope(torch, device, reps=3)
         bench_mla_assemble(torch, device, reps=3)
         print("counter pass done")

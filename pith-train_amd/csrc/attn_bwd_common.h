@@ -66,8 +66,8 @@ void launch_dkdv_d128(const BwdParams& p, bool causal, bool f32_out, unsigned gr
 // dQ for head dims (128, 128): attn_bwd_dq_d128.hip. p.tiles = number of 256-row query tiles.
 void launch_dq_d128(const BwdParams& p, bool causal, bool f32_out, hipStream_t stream);
 
-// dQ for head dims (128, 128) and (192, 128) with 128-row workgroups: attn_bwd_dq_direct.hip.
-// p.tiles = number of 128-row query tiles.
+// dQ for head dims (128, 128) and (192, 128) with 128-row workgroups, early / late wave roles:
+// attn_bwd_dq_direct.hip. p.tiles = number of 128-row query tiles.
 void launch_dq_direct(const BwdParams& p, int dqk, bool causal, bool f32_out, hipStream_t stream);
 
 // Argument checks common to both entry points; returns PITH_OK or records the error.

@@ -303,11 +303,11 @@ extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t strea
   const BwdParams p = make_bwd_params(a);
   hipStream_t st = (hipStream_t)stream;
   begin_launch();
-  const bool half = prefer_half_rows(a->Sq, a->Hq, a->B, a->causal != 0);
-  if ((a->Dqk == 128 && half) || a->Dqk == 192) {
-    // 128-row workgroups whose wave pairs split every tile's keys: the only direct-load form for
-    // 192-feature queries, and the better one for 128 features when 256-row workgroups would
-    // leave compute units idle
+  const bool half = a->Dqk == 192 || prefer_half_rows(a->Sq, a->Hq, a->B, a->causal != 0);
+  if (a->Dqk == 192 || (a->Dqk == 128 && half)) {
+    // early / late wave roles with 128-row workgroups whose wave pairs split every tile's keys: the
+    // only direct-load form for 192-feature queries, and the better one for 128 features when
+    // 256-row workgroups would leave compute units idle
     BwdParams q = p;
     q.tiles = (int)((a->Sq + 127) / 128);
     q.accumulate = a->accumulate_dq;

@@ -81,15 +81,19 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
     delta_q = (p.delta + b * p.lse_bs + (int64_t)h * p.lse_hs)[row];
   }
 
-  // per-lane read offsets inside a tile
-  int s_off[KS];     // straight fragment of tile row c, contraction step ks (+ 32 rows: + 8192 bytes)
-  int t_off[DB][2];  // transposing reads of feature block o, lower / upper 8 rows (+ 16 rows: + 4096 bytes)
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) s_off[ks] = straight_offset128(c, 2 * ks + g);
-#pragma unroll
-  for (int o = 0; o < DB; ++o)
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) t_off[o][hh] = transposed_offset128(0, hh, 32 * o, lane);
+  // per-lane read offsets inside a tile. The swizzle is an XOR on the 16-byte piece index, so the
+  // offsets of the other contraction steps / feature blocks are the first one XOR a constant; only
+  // the first ones live in registers (the kernel sits at the 256-register limit, and a spilled
+  // value is reloaded from scratch with a wait that also waits for the tile loads in flight):
+  //   straight fragment of tile row c, contraction step ks (+ 32 rows: + 8192 bytes):  s_base ^ (ks << 5)
+  //   transposing reads of feature block o, lower / upper 8 rows (+ 16 rows: + 4096 bytes):  t_base[hh] ^ (o << 6)
+  int s_base = straight_offset128(c, g);
+  int t_base[2] = {transposed_offset128(0, 0, 0, lane), transposed_offset128(0, 1, 0, lane)};
+  // called once per interval: the bases are handed to the compiler as new values, or it would
+  // compute every derived offset once and keep all of them in registers across the loop
+  auto refresh_offsets = [&]() __attribute__((always_inline)) { asm volatile("" : "+v"(s_base), "+v"(t_base[0]), "+v"(t_base[1])); };
+  auto s_off = [&](int ks) __attribute__((always_inline)) { return s_base ^ (ks << 5); };
+  auto t_off = [&](int o, int hh) __attribute__((always_inline)) { return t_base[hh] ^ (o << 6); };
 
   f32x16 acc[DB];
 #pragma unroll
@@ -113,14 +117,14 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(ktile + s_off[ks] + nb * 32 * kRowBytes128);
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(ktile + s_off(ks) + nb * 32 * kRowBytes128);
         s[nb] = mfma32(a, qf[ks], s[nb]);
       }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vtile + s_off[ks] + nb * 32 * kRowBytes128);
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vtile + s_off(ks) + nb * 32 * kRowBytes128);
         dp[nb] = mfma32(a, dof[ks], dp[nb]);
       }
   };
@@ -132,7 +136,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
 #pragma unroll
       for (int o = 0; o < DB; ++o) {
         const char* base = ktile + j * 16 * kRowBytes128;
-        at[j][o] = lds_read_transposed_at(base + t_off[o][0], base + t_off[o][1]);
+        at[j][o] = lds_read_transposed_at(base + t_off(o, 0), base + t_off(o, 1));
       }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -176,8 +180,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
     uint32_t w[8];
 #pragma unroll
     for (int ks = 0; ks < kPre; ++ks) {
-      ak[ks] = *reinterpret_cast<const bf16x8*>(ktile + s_off[ks] + nb * 32 * kRowBytes128);
-      av[ks] = *reinterpret_cast<const bf16x8*>(vtile + s_off[ks] + nb * 32 * kRowBytes128);
+      ak[ks] = *reinterpret_cast<const bf16x8*>(ktile + s_off(ks) + nb * 32 * kRowBytes128);
+      av[ks] = *reinterpret_cast<const bf16x8*>(vtile + s_off(ks) + nb * 32 * kRowBytes128);
     }
     f32x16 sn, dn;
 #pragma unroll
@@ -189,8 +193,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + kPre < KS) {
-        ak[ks + kPre] = *reinterpret_cast<const bf16x8*>(ktile + s_off[ks + kPre] + nb * 32 * kRowBytes128);
-        av[ks + kPre] = *reinterpret_cast<const bf16x8*>(vtile + s_off[ks + kPre] + nb * 32 * kRowBytes128);
+        ak[ks + kPre] = *reinterpret_cast<const bf16x8*>(ktile + s_off(ks + kPre) + nb * 32 * kRowBytes128);
+        av[ks + kPre] = *reinterpret_cast<const bf16x8*>(vtile + s_off(ks + kPre) + nb * 32 * kRowBytes128);
       }
       sn = mfma32(ak[ks], qf[ks], sn);
       dn = mfma32(av[ks], dof[ks], dn);
@@ -240,6 +244,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
   end_interval();
   int i = 1;
   for (; i < n_fast; ++i) {  // tiles i-1 and i unmasked
+    refresh_offsets();
     // tile i+1 is requested first: its slots were last read in interval i-1, and the load then
     // has the whole interval to land
     if (i + 1 < n_tiles_wg) request(i + 1);
@@ -252,6 +257,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
     end_interval();
   }
   for (; i < n_tiles_wave; ++i) {  // near the diagonal / ragged end: plain order, masks applied
+    refresh_offsets();
     if (i + 1 < n_tiles_wg) request(i + 1);
     make_ds_half_masked(i - 1, 1);
     accumulate(kslot(i - 1));

@@ -1,18 +1,22 @@
-// Query-gradient kernel with 128-row workgroups for head dims (128, 128) and (192, 128) on gfx950.
+// Query-gradient kernel for head dims (128, 128) and (192, 128) on gfx950, organised like the
+// direct-load forward kernel (256-row workgroups, or 128-row ones whose wave pairs split the keys).
 // Same function and numerics as the other dQ kernels (pithtrain/operators/mla/triton.py:205-266,
 // :392-441: P = exp2(kappa*s - lse2) in fp32, masked entries 0, dS = P*(dP - delta)*scale rounded
 // to bf16, fp32 accumulation of dQ += dS K; `scale` is applied once to the accumulated dQ).
 //
-// Organisation: that of the direct-load forward kernel in its 128-row form (attn_fwd_direct.hip).
-// A workgroup of 8 wavefronts owns 128 query rows of one (batch, head); wave w and wave w + 4 share
-// a SIMD and the SAME 32 query rows (Q^T and dO^T fragments, lse and delta stationary in
-// registers), the early wave (w < 4) owning keys 0-31 and the late wave keys 32-63 of every 64-key
-// tile. K/V tiles go global -> LDS directly into packed swizzled tiles (rings of four, requested
-// two intervals ahead). Per interval a wave runs one matrix block
+// Organisation: that of the direct-load forward kernel (attn_fwd_direct.hip). K/V tiles go
+// global -> LDS directly into packed swizzled tiles (rings of four, requested two intervals ahead).
+// Wave w and wave w + 4 of a workgroup share a SIMD. Per interval a wave runs one matrix block
 //     dQ^T += K(i)^T dS(i)^T ;  S(i+1)^T = K(i+1) Q^T ;  dP(i+1)^T = V(i+1) dO^T
-// and one vector block  dS(i+1) = P o (dP - delta);  early waves run matrix then vector, late waves
-// vector then matrix, so that on every SIMD one wave's MFMAs coincide with the other's arithmetic.
-// At the end the late wave hands its partial dQ to the early wave through LDS.
+// and one vector block  dS(i+1) = P o (dP - delta);  early waves (0-3) run matrix then vector, late
+// waves (4-7) vector then matrix, so that on every SIMD one wave's MFMAs coincide with the other's
+// arithmetic. Q^T and dO^T fragments, lse and delta of a wave's 32 query rows are stationary.
+// FULL: a workgroup owns 256 query rows, every wave 32 of them and all 64 keys of each tile (48
+// matrix instructions per wave and interval against some 110 vector instructions: the vector block
+// hides completely behind the sibling's matrix block).
+// HALF: a workgroup owns 128 query rows; wave w and w + 4 own the SAME 32 rows, the early wave keys
+// 0-31 and the late wave keys 32-63 of every tile; at the end the late wave hands its partial dQ to
+// the early wave through LDS.
 //
 // With 192-feature queries the stationary fragments alone (Q^T 48 + dO^T 32 registers) push a wave
 // past 256 registers, and spilled fragments are reloaded from scratch memory in every interval. The
@@ -33,16 +37,17 @@ namespace {
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
-constexpr int kBM = 128;   // query rows per workgroup
 constexpr int kBN = 64;    // keys per tile
 constexpr int kDv = 128;
 constexpr int kSlots = 4;  // K ring depth (tiles i, i+1 in use, later ones landing); a power of two
 constexpr int kAhead = 4;  // fragment reads run this many products ahead in the matrix block
 constexpr int kTile = kBN * kRowBytes128;
 
-template <int DQK, bool CAUSAL, typename OutT>
+template <int DQK, bool HALF, bool CAUSAL, typename OutT>
 __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams p) {
-  static_assert(DQK == 128 || DQK == 192, "head dims");
+  static_assert(DQK == 128 || (DQK == 192 && HALF), "head dims (192-feature queries need the HALF form)");
+  constexpr int KVB = HALF ? 1 : 2;      // 32-key blocks of a tile this wave owns
+  constexpr int kBM = HALF ? 128 : 256;  // query rows per workgroup
   // kDist: a tile is requested kDist intervals before the interval that first reads it.
   // kLdsQ / kLdsDo: trailing Q^T / dO^T fragments kept in LDS instead of registers.
   constexpr int kDist = DQK == 192 ? 1 : 2;
@@ -62,13 +67,13 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, g = lane >> 5;
   const bool late = wave >= kWaves / 2;
-  const int kvb0 = wave >> 2;  // the 32-key block of every tile this wave owns
+  const int kvb0 = HALF ? wave >> 2 : 0;  // the first 32-key block of every tile this wave owns
 
   int m_tile, h, b;
   decode_block(blockIdx.x, p.Hq, p.B, p.tiles, m_tile, h, b);
   const int hk = h / p.group;
   const int m0 = m_tile * kBM;
-  const int q_wave0 = m0 + (wave & 3) * 32;
+  const int q_wave0 = m0 + (HALF ? (wave & 3) : wave) * 32;
   const int qrow = q_wave0 + c;
 
   const int64_t q_row_stride = (int64_t)p.Hq * DQK;
@@ -143,25 +148,32 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
     return ks < VSR ? dof[ks < VSR ? ks : 0] : *reinterpret_cast<const bf16x8*>(stat + (kLdsQ + ks - VSR) * 1024);
   };
 
-  // per-lane read offsets inside a tile, for this wave's key block
-  // s_off[ks]: straight fragment of key row c, contraction step ks: steps 0..7 in the 128-feature
-  // tile (K and V), steps 8.. in the extra tile behind the K tile.
-  // t_off[o][hh]: transposing reads of K feature block o, lower / upper 8 keys of a 16-key step
-  // (+ 16 keys: + 4096 bytes): blocks 0..3 in the 128-feature tile, 4.. in the extra tile.
-  int s_off[KS];
-  int t_off[DB][2];
+  // per-lane read offsets inside a tile, for this wave's key block. The swizzle is an XOR on the
+  // 16-byte piece index, so the offsets of all contraction steps / feature blocks of one tile part
+  // differ from the first one by an XOR with a constant: only the first ones are kept in registers
+  // (s_base / t_base: 128-feature tile, sx_base / tx_base: the extra tile behind a K tile).
+  //   straight fragment of key row c, contraction step ks:  s_base ^ (ks << 5)      (ks < 8)
+  //                                                          sx_base ^ ((ks-8) << 5) (ks >= 8)
+  //   transposing reads of K feature block o, lower / upper 8 keys of a 16-key step (+ 16 keys:
+  //   + 4096 bytes):  t_base[hh] ^ (o << 6)  (o < 4),  tx_base[hh] ^ ((o-4) << 6)  (o >= 4)
+  int s_base = straight_offset128(c, g) + kvb0 * 32 * kRowBytes128;
+  int sx_base = kTile + straight_offset128(c, g + 8 * kvb0);
+  int t_base[2], tx_base[2];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    if (ks < 8) s_off[ks] = straight_offset128(c, 2 * ks + g) + kvb0 * 32 * kRowBytes128;
-    else s_off[ks] = kTile + straight_offset128(c, 2 * (ks - 8) + g + 8 * kvb0);
+  for (int hh = 0; hh < 2; ++hh) {
+    t_base[hh] = transposed_offset128(0, hh, 0, lane) + kvb0 * 32 * kRowBytes128;
+    tx_base[hh] = kTile + transposed_offset128(0, hh, 64 * kvb0, lane);
   }
-#pragma unroll
-  for (int o = 0; o < DB; ++o)
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-      if (o < 4) t_off[o][hh] = transposed_offset128(0, hh, 32 * o, lane) + kvb0 * 32 * kRowBytes128;
-      else t_off[o][hh] = kTile + transposed_offset128(0, hh, 64 * kvb0 + 32 * (o - 4), lane);
-    }
+  // Called once per interval: the compiler must take the base offsets as new values each time, or it
+  // would compute all derived offsets once, keep them in registers across the loop and spill others.
+  auto refresh_offsets = [&]() __attribute__((always_inline)) {
+    if constexpr (DQK == 192) asm volatile("" : "+v"(s_base), "+v"(sx_base), "+v"(t_base[0]), "+v"(t_base[1]), "+v"(tx_base[0]), "+v"(tx_base[1]));
+    else if constexpr (!HALF) asm volatile("" : "+v"(s_base), "+v"(t_base[0]), "+v"(t_base[1]));
+  };
+  auto s_off = [&](int ks) __attribute__((always_inline)) { return ks < 8 ? s_base ^ (ks << 5) : sx_base ^ ((ks - 8) << 5); };
+  auto t_off = [&](int o, int hh) __attribute__((always_inline)) {
+    return o < 4 ? t_base[hh] ^ (o << 6) : tx_base[hh] ^ ((o - 4) << 6);
+  };
 
   f32x16 acc[DB];
 #pragma unroll
@@ -169,76 +181,98 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
 
-  f32x16 s, dp;   // S^T and dP^T of this wave's 32 keys of one tile: [keys] x [queries]
-  bf16x8 dsf[2];  // dS^T / scale of the same keys as B operand, one fragment per 16 keys
+  f32x16 s[KVB], dp[KVB];  // S^T and dP^T of this wave's keys of one tile: 32 x 32 tiles [keys] x [queries]
+  bf16x8 dsf[2 * KVB];     // dS^T / scale of the same keys as B operand, one fragment per 16 keys
+  // straight fragment of key block kvb: the 128-feature tile steps 32 rows on, the extra tile (192
+  // features, HALF only) is never asked for a second block
+  auto a_frag = [&](const char* tile, int ks, int kvb) __attribute__((always_inline)) {
+    return *reinterpret_cast<const bf16x8*>(tile + s_off(ks) + kvb * 32 * kRowBytes128);
+  };
 
   // ---- S^T = K Q^T and dP^T = V dO^T
   auto scores = [&](const char* ktile, const char* vtile) __attribute__((always_inline)) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      s[v] = 0.f;
-      dp[v] = 0.f;
-    }
+    for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) s = mfma32(*reinterpret_cast<const bf16x8*>(ktile + s_off[ks]), q_frag(ks), s);
+      for (int v = 0; v < 16; ++v) {
+        s[kvb][v] = 0.f;
+        dp[kvb][v] = 0.f;
+      }
 #pragma unroll
-    for (int ks = 0; ks < VS; ++ks) dp = mfma32(*reinterpret_cast<const bf16x8*>(vtile + s_off[ks]), do_frag(ks), dp);
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int kvb = 0; kvb < KVB; ++kvb) s[kvb] = mfma32(a_frag(ktile, ks, kvb), q_frag(ks), s[kvb]);
+#pragma unroll
+    for (int ks = 0; ks < VS; ++ks)
+#pragma unroll
+      for (int kvb = 0; kvb < KVB; ++kvb) dp[kvb] = mfma32(a_frag(vtile, ks, kvb), do_frag(ks), dp[kvb]);
   };
   // ---- dQ^T += K^T dS^T
   auto accumulate = [&](const char* ktile) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 2 * KVB; ++j)
 #pragma unroll
       for (int o = 0; o < DB; ++o) {
         const char* base = ktile + j * 16 * kRowBytes128;
-        acc[o] = mfma32(lds_read_transposed_at(base + t_off[o][0], base + t_off[o][1]), dsf[j], acc[o]);
+        acc[o] = mfma32(lds_read_transposed_at(base + t_off(o, 0), base + t_off(o, 1)), dsf[j], acc[o]);
       }
   };
   // ---- matrix block: the gradient product of tile `kprev`, then both score products of the next
   // tile: first the contraction steps whose B operand sits in registers, then those whose B operand
   // is read from LDS (two reads per product, like the transposed fragments).
   auto matrix_block = [&](const char* kprev, const char* ktile, const char* vtile) __attribute__((always_inline)) {
-    constexpr int NT = 2 * DB, N1 = KSR + VSR, N2 = kLdsQ + kLdsDo;
+    constexpr int NT = 2 * KVB * DB, N1 = KVB * (KSR + VSR), N2 = kLdsQ + kLdsDo;
     static_assert(kAhead <= NT && kAhead <= N1 && (N2 == 0 || kAhead <= N2), "look-ahead segments");
-    bf16x8 at[2][DB], ak[KS], av[VS], bq[kLdsQ + 1], bd[kLdsDo + 1];
+    static_assert(N2 == 0 || KVB == 1, "LDS-resident B operands only in the HALF form");
+    bf16x8 at[2 * KVB][DB], ak[KS][KVB], av[VS][KVB], bq[kLdsQ + 1], bd[kLdsDo + 1];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 2 * KVB; ++j)
 #pragma unroll
       for (int o = 0; o < DB; ++o) {
         const char* base = kprev + j * 16 * kRowBytes128;
-        at[j][o] = lds_read_transposed_at(base + t_off[o][0], base + t_off[o][1]);
+        at[j][o] = lds_read_transposed_at(base + t_off(o, 0), base + t_off(o, 1));
       }
 #pragma unroll
-    for (int ks = 0; ks < KSR; ++ks) ak[ks] = *reinterpret_cast<const bf16x8*>(ktile + s_off[ks]);
+    for (int ks = 0; ks < KSR; ++ks)
 #pragma unroll
-    for (int ks = 0; ks < VSR; ++ks) av[ks] = *reinterpret_cast<const bf16x8*>(vtile + s_off[ks]);
+      for (int kvb = 0; kvb < KVB; ++kvb) ak[ks][kvb] = a_frag(ktile, ks, kvb);
+#pragma unroll
+    for (int ks = 0; ks < VSR; ++ks)
+#pragma unroll
+      for (int kvb = 0; kvb < KVB; ++kvb) av[ks][kvb] = a_frag(vtile, ks, kvb);
 #pragma unroll
     for (int ks = 0; ks < kLdsQ; ++ks) {
-      ak[KSR + ks] = *reinterpret_cast<const bf16x8*>(ktile + s_off[KSR + ks]);
+      ak[KSR + ks][0] = a_frag(ktile, KSR + ks, 0);
       bq[ks] = *reinterpret_cast<const bf16x8*>(stat + ks * 1024);
     }
 #pragma unroll
     for (int ks = 0; ks < kLdsDo; ++ks) {
-      av[VSR + ks] = *reinterpret_cast<const bf16x8*>(vtile + s_off[VSR + ks]);
+      av[VSR + ks][0] = a_frag(vtile, VSR + ks, 0);
       bd[ks] = *reinterpret_cast<const bf16x8*>(stat + (kLdsQ + ks) * 1024);
     }
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 2 * KVB; ++j)
 #pragma unroll
       for (int o = 0; o < DB; ++o) acc[o] = mfma32(at[j][o], dsf[j], acc[o]);
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      s[v] = 0.f;
-      dp[v] = 0.f;
-    }
+    for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
-    for (int ks = 0; ks < KSR; ++ks) s = mfma32(ak[ks], qf[ks], s);
+      for (int v = 0; v < 16; ++v) {
+        s[kvb][v] = 0.f;
+        dp[kvb][v] = 0.f;
+      }
 #pragma unroll
-    for (int ks = 0; ks < VSR; ++ks) dp = mfma32(av[ks], dof[ks], dp);
+    for (int ks = 0; ks < KSR; ++ks)
 #pragma unroll
-    for (int ks = 0; ks < kLdsQ; ++ks) s = mfma32(ak[KSR + ks], bq[ks], s);
+      for (int kvb = 0; kvb < KVB; ++kvb) s[kvb] = mfma32(ak[ks][kvb], qf[ks], s[kvb]);
 #pragma unroll
-    for (int ks = 0; ks < kLdsDo; ++ks) dp = mfma32(av[VSR + ks], bd[ks], dp);
+    for (int ks = 0; ks < VSR; ++ks)
+#pragma unroll
+      for (int kvb = 0; kvb < KVB; ++kvb) dp[kvb] = mfma32(av[ks][kvb], dof[ks], dp[kvb]);
+#pragma unroll
+    for (int ks = 0; ks < kLdsQ; ++ks) s[0] = mfma32(ak[KSR + ks][0], bq[ks], s[0]);
+#pragma unroll
+    for (int ks = 0; ks < kLdsDo; ++ks) dp[0] = mfma32(av[VSR + ks][0], bd[ks], dp[0]);
     // Reads run kAhead products ahead: after product m come the reads of product m + kAhead.
     // Products 0 .. NT-1 and the last N2 take two LDS reads each, the N1 in between one.
     __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
@@ -263,20 +297,27 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   auto make_ds = [&](int t) __attribute__((always_inline)) {
     const int n0 = t * kBN;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) s[v] = __builtin_amdgcn_exp2f(s[v] * p.kappa - lse_q);
+    for (int kvb = 0; kvb < KVB; ++kvb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[kvb][v] = __builtin_amdgcn_exp2f(s[kvb][v] * p.kappa - lse_q);
     if ((CAUSAL && (n0 + kBN - 1 > q_wave0)) || (n0 + kBN > p.Skv)) {
       // tile crossing the diagonal of a causal chunk, or a ragged last tile (wave-uniform branch)
       const int limit = CAUSAL ? min(qrow, p.Skv - 1) : p.Skv - 1;  // last visible key
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        if (n0 + kvb0 * 32 + acc_row(v, g) > limit) s[v] = 0.f;
+      for (int kvb = 0; kvb < KVB; ++kvb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (n0 + (kvb0 + kvb) * 32 + acc_row(v, g) > limit) s[kvb][v] = 0.f;
     }
 #pragma unroll
-    for (int v = 0; v < 16; ++v) s[v] *= dp[v] - delta_q;
+    for (int kvb = 0; kvb < KVB; ++kvb) {
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj)
-      dsf[jj] = to_bf16x8(s[8 * jj], s[8 * jj + 1], s[8 * jj + 2], s[8 * jj + 3], s[8 * jj + 4], s[8 * jj + 5],
-                          s[8 * jj + 6], s[8 * jj + 7]);
+      for (int v = 0; v < 16; ++v) s[kvb][v] *= dp[kvb][v] - delta_q;
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+        dsf[2 * kvb + jj] = to_bf16x8(s[kvb][8 * jj], s[kvb][8 * jj + 1], s[kvb][8 * jj + 2], s[kvb][8 * jj + 3],
+                                      s[kvb][8 * jj + 4], s[kvb][8 * jj + 5], s[kvb][8 * jj + 6], s[kvb][8 * jj + 7]);
+    }
   };
 
   // Every interval ends by waiting until at most the loads of the last kDist - 1 intervals are
@@ -305,6 +346,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   auto interval = [&](int i, auto late_tag, auto full_tag) __attribute__((always_inline)) {
     constexpr bool LATE = decltype(late_tag)::value, FULL = decltype(full_tag)::value;
     const bool will_request = i + 1 + kDist < n_tiles_wg;
+    refresh_offsets();
     if (!LATE) {
       if (FULL) {
         matrix_block(kslot(i), kslot(i + 1), vslot(i + 1));
@@ -338,6 +380,19 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   // wave passed the barrier that ends the last interval)
   constexpr int kExch = DB * 4 * 64 * 16;
   char* const exch = smem + (wave & 3) * kExch;
+  if constexpr (!HALF) {
+    OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * DQK;
+    if (qrow < p.Sq) {
+      OutT* dst = dqh + qrow * q_row_stride;
+#pragma unroll
+      for (int o = 0; o < DB; ++o)
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4)
+          store4<OutT>(dst + 32 * o + 8 * b4 + 4 * g, acc[o][4 * b4] * p.scale, acc[o][4 * b4 + 1] * p.scale,
+                       acc[o][4 * b4 + 2] * p.scale, acc[o][4 * b4 + 3] * p.scale, p.accumulate != 0);
+    }
+    return;
+  }
   if (late) {
 #pragma unroll
     for (int o = 0; o < DB; ++o)
@@ -364,23 +419,25 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   }
 }
 
-template <int DQK>
+template <int DQK, bool HALF>
 void launch_one(const BwdParams& p, bool causal, bool f32_out, hipStream_t st) {
   const dim3 grid((unsigned)(p.tiles * p.Hq * p.B)), block(kThreads);
   if (causal) {
-    if (f32_out) hipLaunchKernelGGL((attn_bwd_dq_direct_kernel<DQK, true, float>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((attn_bwd_dq_direct_kernel<DQK, true, __bf16>), grid, block, 0, st, p);
+    if (f32_out) hipLaunchKernelGGL((attn_bwd_dq_direct_kernel<DQK, HALF, true, float>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((attn_bwd_dq_direct_kernel<DQK, HALF, true, __bf16>), grid, block, 0, st, p);
   } else {
-    if (f32_out) hipLaunchKernelGGL((attn_bwd_dq_direct_kernel<DQK, false, float>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((attn_bwd_dq_direct_kernel<DQK, false, __bf16>), grid, block, 0, st, p);
+    if (f32_out) hipLaunchKernelGGL((attn_bwd_dq_direct_kernel<DQK, HALF, false, float>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((attn_bwd_dq_direct_kernel<DQK, HALF, false, __bf16>), grid, block, 0, st, p);
   }
 }
 
 }  // namespace
 
 void launch_dq_direct(const BwdParams& p, int dqk, bool causal, bool f32_out, hipStream_t st) {
-  if (dqk == 128) launch_one<128>(p, causal, f32_out, st);
-  else launch_one<192>(p, causal, f32_out, st);
+  // only the HALF form is built: with all 64 keys of a tile per wave this organisation needs some 300
+  // registers (the 256-row kernel for 128 features is attn_bwd_dq_d128.hip, organised differently)
+  if (dqk == 192) launch_one<192, true>(p, causal, f32_out, st);
+  else launch_one<128, true>(p, causal, f32_out, st);
 }
 
 }  // namespace pith

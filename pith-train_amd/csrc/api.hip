@@ -38,7 +38,7 @@ int compute_units() {
 // work, so a launch needs about four rounds of workgroups before the light ones fill the gaps;
 // without a mask only the fill of the last round matters.
 bool prefer_half_rows(int64_t Sq, int64_t Hq, int64_t B, bool causal) {
-  const int64_t cus = compute_units() > 0 ? compute_units() : 256;
+  const int64_t cus = compute_units_or_default();
   const int64_t wgs = ((Sq + 255) / 256) * Hq * B;
   if (causal) return wgs < 4 * cus;
   const int64_t rounds = (wgs + cus - 1) / cus;

@@ -315,7 +315,8 @@ int pick_split(const pith_attn_bwd_args* a) {
   const int64_t group = a->Hq / a->Hkv;
   const int64_t base = ((a->Skv + kBN - 1) / kBN) * a->Hkv * a->B;
   int split = 1;
-  while (split < group && base * split < 512 && group % (split * 2) == 0) split *= 2;
+  const int64_t want = 2 * (int64_t)compute_units_or_default();  // two rounds of workgroups
+  while (split < group && base * split < want && group % (split * 2) == 0) split *= 2;
   return split;
 }
 

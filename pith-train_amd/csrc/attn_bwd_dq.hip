@@ -316,7 +316,7 @@ extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t strea
     launch_dq<128, 128, 1, 2, 8>(p, a, st);
   } else {
     // short query ranges: workgroups of 4 wavefronts x 32 rows, so that no compute unit idles
-    const bool few = ((a->Sq + 255) / 256) * a->Hq * a->B < 192;
+    const bool few = ((a->Sq + 255) / 256) * a->Hq * a->B * 4 < 3 * (int64_t)compute_units_or_default();
     if (few) launch_dq<64, 64, 1, 1, 4>(p, a, st);
     else launch_dq<64, 64, 1, 1, 8>(p, a, st);
   }

@@ -246,9 +246,11 @@ void launch_fwd(FwdParams p, const pith_attn_fwd_args* a, hipStream_t st) {
 }
 
 // With 256 query rows per workgroup a short query range leaves compute units idle (one workgroup
-// per unit at these LDS sizes): below 3/4 of the device's 256 units the launch uses workgroups
+// per unit at these LDS sizes): below 3/4 of the device's compute units the launch uses workgroups
 // of 4 wavefronts x 32 rows instead, which doubles their number.
-bool few_workgroups(int64_t Sq, int64_t Hq, int64_t B) { return ((Sq + 255) / 256) * Hq * B < 192; }
+bool few_workgroups(int64_t Sq, int64_t Hq, int64_t B) {
+  return ((Sq + 255) / 256) * Hq * B * 4 < 3 * (int64_t)compute_units_or_default();
+}
 
 }  // namespace
 }  // namespace pith

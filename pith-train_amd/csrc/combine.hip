@@ -397,7 +397,8 @@ __global__ __launch_bounds__(256) void cast_f32_bf16_kernel(const float* __restr
 // Rows per block: as many as keep the grid at several blocks per CU and the LDS patch small.
 int pick_tile_s(int64_t B, int64_t S, int64_t H, int max_rows) {
   int ts = 16;
-  while (ts > 1 && (B * ((S + ts - 1) / ts) < 2048 || ts * H > max_rows)) ts >>= 1;
+  const int64_t want = 8 * (int64_t)compute_units_or_default();  // eight resident blocks per compute unit
+  while (ts > 1 && (B * ((S + ts - 1) / ts) < want || ts * H > max_rows)) ts >>= 1;
   return ts;
 }
 

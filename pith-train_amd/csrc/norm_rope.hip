@@ -338,7 +338,8 @@ Plan make_plan(int64_t B, int64_t S, int64_t H, int64_t D) {
   const int slots = kThreads / pl.lanes;
   int hg = 1;
   while (hg < slots && hg * 8 < H) hg <<= 1;
-  while (hg < slots && hg < H && B * ((S * hg + slots - 1) / slots) < 2048) hg <<= 1;
+  const int64_t want = 8 * (int64_t)compute_units_or_default();  // eight resident blocks per compute unit
+  while (hg < slots && hg < H && B * ((S * hg + slots - 1) / slots) < want) hg <<= 1;
   pl.hg = hg;
   pl.tile_s = slots / hg;
   pl.n_tiles = (int)((S + pl.tile_s - 1) / pl.tile_s);

@@ -19,6 +19,11 @@ int check_launch(const char* what);
 
 // Compute units of the current device (looked up once per device; 0 if the runtime cannot tell).
 int compute_units();
+// The same for launch heuristics: 256 (an MI355X) when the runtime cannot tell.
+inline int compute_units_or_default() {
+  const int n = compute_units();
+  return n > 0 ? n : 256;
+}
 
 // Work split of the query-stationary direct-load kernels (forward, dQ): true = 128-row workgroups.
 bool prefer_half_rows(int64_t Sq, int64_t Hq, int64_t B, bool causal);

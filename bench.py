@@ -2,6 +2,7 @@
 """Benchmark of the ring-attention hot path on ONE MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra-configs]
+    python bench.py --config mla16k|long131k [--steps K]     (one of the other configurations alone)
 
 A step is one forward + backward pass of one GPU's share of causal ring attention at the
 Qwen3-30B-A3B shape (32 q heads / 4 kv heads, head dim 128, 32768 tokens as 4 zigzag chunks of 8192,
@@ -385,6 +386,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-configs", action="store_true",
                     help="skip the MLA 16K and long 131K configurations (sub-objects mla16k, long131k)")
+    ap.add_argument("--config", choices=["mla16k", "long131k"], default=None,
+                    help="time only this configuration's ring share and print its sub-object (for kernel traces)")
     ap.add_argument("--counter-pass", action="store_true",
                     help="run only the roofline kernel and a calibration copy (for rocprofv3 --pmc), print no JSON")
     args = ap.parse_args()
@@ -400,6 +403,10 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.config:
+        cfg = MLA16K if args.config == "mla16k" else LONG131K
+        print(json.dumps({args.config: bench_other_config(torch, device, cfg, args.steps, args.warmup)}))
+        return
     host_inputs, dev_inputs = make_inputs(torch, device)
     ring = bench_ring(torch, args, dev_inputs)
     if ring is None:

@@ -294,13 +294,16 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
     __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
   };
   // ---- s, dp of tile t -> dS / scale as bf16 fragments
-  auto make_ds = [&](int t) __attribute__((always_inline)) {
+  // MASKED = false: the caller knows that tile t lies entirely below this wave's diagonal and inside
+  // the key range (no mask code, and nothing it needs stays live in the loop that uses it)
+  auto make_ds = [&](int t, auto masked_tag) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
     const int n0 = t * kBN;
 #pragma unroll
     for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) s[kvb][v] = __builtin_amdgcn_exp2f(s[kvb][v] * p.kappa - lse_q);
-    if ((CAUSAL && (n0 + kBN - 1 > q_wave0)) || (n0 + kBN > p.Skv)) {
+    if (MASKED && ((CAUSAL && (n0 + kBN - 1 > q_wave0)) || (n0 + kBN > p.Skv))) {
       // tile crossing the diagonal of a causal chunk, or a ragged last tile (wave-uniform branch)
       const int limit = CAUSAL ? min(qrow, p.Skv - 1) : p.Skv - 1;  // last visible key
 #pragma unroll
@@ -336,14 +339,16 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far, the stationary fragments included
   __syncthreads();
   scores(kslot(0), vslot(0));
-  if (!late) make_ds(0);
+  if (!late) make_ds(0, std::true_type{});
 
   // Interval i = 0 .. n_tiles_wg - 1 reads K(i) (gradient product), K(i+1) and V(i+1) (scores) and
   // requests tile i + 1 + kDist, whose slots were last read in interval i - 1 (kDist 2: they held
   // tile i - 1) or hold nothing that is still needed (kDist 1: K slot of tile i - 2, V slot of tile i,
   // read in interval i - 1).
   // FULL: this wave has both a tile to accumulate and a next tile to score.
-  auto interval = [&](int i, auto late_tag, auto full_tag) __attribute__((always_inline)) {
+  // MASKED: the tile whose dS this interval makes (i + 1 in the early waves, i in the late ones) may
+  // need the mask.
+  auto interval = [&](int i, auto late_tag, auto full_tag, auto masked_tag) __attribute__((always_inline)) {
     constexpr bool LATE = decltype(late_tag)::value, FULL = decltype(full_tag)::value;
     const bool will_request = i + 1 + kDist < n_tiles_wg;
     refresh_offsets();
@@ -352,28 +357,35 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
         matrix_block(kslot(i), kslot(i + 1), vslot(i + 1));
         __builtin_amdgcn_sched_barrier(0);
         if (will_request) request(i + 1 + kDist);
-        make_ds(i + 1);
+        make_ds(i + 1, masked_tag);
       } else {
         if (i < n_tiles_wave) accumulate(kslot(i));
         if (will_request) request(i + 1 + kDist);
       }
     } else {
       if (will_request) request(i + 1 + kDist);
-      if (FULL || i < n_tiles_wave) make_ds(i);
+      if (FULL || i < n_tiles_wave) make_ds(i, masked_tag);
       __builtin_amdgcn_sched_barrier(0);
       if (FULL) matrix_block(kslot(i), kslot(i + 1), vslot(i + 1));
       else if (i < n_tiles_wave) accumulate(kslot(i));
     }
     land_and_sync(will_request);
   };
+  // tiles [0, first_masked) need no mask for this wave: they lie below its diagonal and inside Skv
+  int first_masked = p.Skv / kBN;
+  if (CAUSAL) first_masked = min(first_masked, q_wave0 >= kBN - 1 ? (q_wave0 - (kBN - 1)) / kBN + 1 : 0);
+  constexpr std::false_type no;
+  constexpr std::true_type yes;
   if (!late) {
     int i = 0;
-    for (; i + 1 < n_tiles_wave; ++i) interval(i, std::false_type{}, std::true_type{});
-    for (; i < n_tiles_wg; ++i) interval(i, std::false_type{}, std::false_type{});
+    for (; i + 1 < min(n_tiles_wave, first_masked); ++i) interval(i, no, yes, no);  // makes dS(i + 1)
+    for (; i + 1 < n_tiles_wave; ++i) interval(i, no, yes, yes);
+    for (; i < n_tiles_wg; ++i) interval(i, no, no, yes);
   } else {
     int i = 0;
-    for (; i + 1 < n_tiles_wave; ++i) interval(i, std::true_type{}, std::true_type{});
-    for (; i < n_tiles_wg; ++i) interval(i, std::true_type{}, std::false_type{});
+    for (; i + 1 < n_tiles_wave && i < first_masked; ++i) interval(i, yes, yes, no);  // makes dS(i)
+    for (; i + 1 < n_tiles_wave; ++i) interval(i, yes, yes, yes);
+    for (; i < n_tiles_wg; ++i) interval(i, yes, no, yes);
   }
 
   // ---- the late wave of a pair hands its partial dQ to the early wave (the tile ring is free: every

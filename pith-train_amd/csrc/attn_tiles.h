@@ -184,32 +184,38 @@ __device__ __forceinline__ void load_lds4(const void* src, char* dst_wave) {
 }
 
 // Moves a [ROWS x 128] bf16 tile with THREADS threads (THREADS / 64 wavefronts): wavefront w
-// moves the 4 tile rows of every 1 KB region n * WAVES + w.
+// moves the 4 tile rows of every 1 KB region n * WAVES + w. With 4 * WAVES a multiple of 16 the
+// swizzle of a lane's row is the same in every region, so one per-lane source offset serves all
+// regions and the region only moves the (uniform) source address on.
 template <int ROWS, int THREADS>
 struct DirectTile128 {
   static constexpr int kWaves = THREADS / 64;
   static constexpr int kPerThread = ROWS * 16 / THREADS;
   static_assert(ROWS * 16 % THREADS == 0, "tile must split evenly over the threads");
+  static_assert((4 * kWaves) % 16 == 0, "rows of successive regions must share their swizzle");
   static constexpr int kTileBytes = ROWS * kRowBytes128;
-  int src_off[kPerThread];  // byte offset of this lane's source piece from the tile's first row
+  int src_off;  // byte offset of this lane's source piece in region 0 from the tile's first row
   int row_bytes;
 
   // row_bytes: distance between consecutive rows in global memory, in bytes
   __device__ __forceinline__ void init(int row_bytes_, int wave, int lane) {
     row_bytes = row_bytes_;
-#pragma unroll
-    for (int n = 0; n < kPerThread; ++n) {
-      const int row = 4 * (n * kWaves + wave) + (lane >> 4);
-      src_off[n] = row * row_bytes + (((lane & 15) ^ tile_swizzle(row)) << 4);
-    }
+    const int row = 4 * wave + (lane >> 4);
+    src_off = row * row_bytes + (((lane & 15) ^ tile_swizzle(row)) << 4);
   }
   // tile_src: address of [first row of the tile][feature 0] of the head slice (uniform);
   // rows_left: valid rows from there on (>= 1), rows beyond are read from the last valid row.
   // `slot` is the LDS tile (uniform).
   __device__ __forceinline__ void issue(const char* tile_src, int rows_left, char* slot, int wave, int lane) const {
     if (rows_left >= ROWS) {
+      // The offset is pinned in a register BEFORE the first load is issued: were it spilled, the
+      // compiler would reload it between two loads and wait for the reload with a counter wait that
+      // also waits for every tile load issued before it.
+      int off = src_off;
+      asm volatile("" : "+v"(off));
 #pragma unroll
-      for (int n = 0; n < kPerThread; ++n) load_lds16(tile_src, src_off[n], slot + (n * kWaves + wave) * 1024);
+      for (int n = 0; n < kPerThread; ++n)
+        load_lds16(tile_src + (int64_t)n * 4 * kWaves * row_bytes, off, slot + (n * kWaves + wave) * 1024);
     } else {
 #pragma unroll
       for (int n = 0; n < kPerThread; ++n) {

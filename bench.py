@@ -44,7 +44,7 @@ HBM_PEAK_GBPS = 8000.0
 
 HQ, HKV, DQK, DV, S_LOCAL, CP, RANK = 32, 4, 128, 128, 8192, 4, 1
 LAYOUT = "zigzag"
-COMBINE_TRAFFIC = 144_900_000
+COMBINE_TRAFFIC = 135_900_000
 
 
 # Figures that are NOT measured by this program: hardware-counter results of rocprofv3 --pmc runs over
@@ -55,11 +55,11 @@ FROM_PROFILES = {
     "attn_bwd_dkdv_d128_kernel<non-causal>": {
         "file": "profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt",
         "hbm_bytes_per_launch": 282_700_000,  # 215.6 MB fetched + 67.1 MB written (FETCH_SIZE / WRITE_SIZE, calibrated on a copy)
-        "mfma_file": "profiles/attn_d128_kernels_mfma_lds_counters.txt",
-        "mfma_busy_fraction": 0.63,  # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs)
-        "sustained_clock_ghz": 1.87,  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration (2.4 GHz nominal)
+        "mfma_file": "profiles/attn_kernels_mfma_lds_counters.txt",
+        "mfma_busy_fraction": 0.615,  # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs)
+        "sustained_clock_ghz": 1.85,  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration (2.4 GHz nominal)
     },
-    "combine_kernel": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_per_launch": COMBINE_TRAFFIC},
+    "combine_front_kernel": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_per_launch": COMBINE_TRAFFIC},
     "norm_rope_kernels": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_fwd_plus_bwd": 159_400_000 + 235_200_000},
     "mla_assemble_kernels": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_fwd_plus_bwd": 128_000_000 + 128_000_000},
 }
@@ -500,8 +500,8 @@ def main():
             "bytes": comb_bytes,
             "roofline": {"bound": "hbm", "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": round(comb_gbps / HBM_PEAK_GBPS, 4),
-                         "traffic": FROM_PROFILES["combine_kernel"]["hbm_bytes_per_launch"],
-                         "traffic_from": FROM_PROFILES["combine_kernel"]["file"]},
+                         "traffic": FROM_PROFILES["combine_front_kernel"]["hbm_bytes_per_launch"],
+                         "traffic_from": FROM_PROFILES["combine_front_kernel"]["file"]},
             "cpu_baseline": combine_cpu,
         },  # fmt: skip
         "norm_rope": {

@@ -188,6 +188,8 @@ typedef struct {
   int64_t k_pe_bs, k_pe_rs;  /* batch / row strides of k_pe, elements */
   void* dk_pe;               /* pith_attn_bwd_dkdv with k_pe: gradient of k_pe */
   int64_t dk_pe_bs;
+  void* ds;                  /* optional dS hand-over buffer (see below), 256-byte aligned; may be NULL */
+  int64_t ds_bytes;          /* its size */
 } pith_attn_bwd_args;
 
 int pith_attn_bwd_dkdv(const pith_attn_bwd_args* args, pith_stream_t stream);
@@ -200,6 +202,19 @@ int pith_attn_bwd_dq(const pith_attn_bwd_args* args, pith_stream_t stream);
  * smaller one, the call still succeeds and one workgroup walks all heads of a group. The
  * workspace is only used during the call's kernels; nothing is kept in it between calls. */
 int64_t pith_attn_bwd_dkdv_workspace_bytes(const pith_attn_bwd_args* args);
+
+/* dS hand-over between the two backward calls of one chunk (no counterpart in the reference, whose
+ * two kernels each recompute S and dP, mla/triton.py:130-266). When `ds` is set,
+ * pith_attn_bwd_dkdv also stores every dS tile it forms (bf16, in a layout private to the library)
+ * and a pith_attn_bwd_dq call with the SAME shapes, strides, causal flag and `ds`, enqueued after
+ * it on the same stream, computes dQ = scale * dS K from those tiles without recomputing the
+ * scores: the backward then executes 5 matrix products instead of 7, at the price of
+ * Sq*Skv*Hq*B*2 bytes written and read once. Results agree with the recomputing dQ kernel up to
+ * fp32 summation order (the dS values are the same bf16 numbers). The buffer holds nothing of
+ * value after the dQ call. Returns the bytes needed, or 0 when the shape has no hand-over path
+ * (head dims other than (128,128)); with ds == NULL or a buffer that is too small both calls
+ * behave as before. */
+int64_t pith_attn_bwd_ds_bytes(const pith_attn_bwd_args* args);
 
 /* pith_attn_bwd_dkdv for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the

@@ -29,6 +29,10 @@ struct BwdParams {
   const __bf16* k_pe;
   int64_t k_pe_bs, k_pe_rs;
   float* ws_dkpe;
+  // dS hand-over from the dK/dV kernel to the dQ kernel (head dims 128/128): bf16 images, 16 KB per
+  // (batch, query head, 64-row query tile, 128-key block); ds_qt / ds_kb = number of such tiles / blocks
+  char* ds;
+  int ds_qt, ds_kb;
 };
 
 // Stores 4 consecutive output features held by one lane; OutT is __bf16 or float.
@@ -69,6 +73,12 @@ void launch_dq_d128(const BwdParams& p, bool causal, bool f32_out, hipStream_t s
 // dQ for head dims (128, 128) and (192, 128) with 128-row workgroups, early / late wave roles:
 // attn_bwd_dq_direct.hip. p.tiles = number of 128-row query tiles.
 void launch_dq_direct(const BwdParams& p, int dqk, bool causal, bool f32_out, hipStream_t stream);
+
+// dQ for head dims (128, 128) from the dS images the dK/dV kernel left in p.ds: attn_bwd_dq_ds.hip.
+// p.tiles = number of 512-row query tiles.
+void launch_dq_from_ds(const BwdParams& p, bool causal, bool f32_out, hipStream_t stream);
+// Bytes of dS images for a shape (0: the shape has no hand-over path).
+int64_t ds_bytes_for(const pith_attn_bwd_args* a);
 
 // Argument checks common to both entry points; returns PITH_OK or records the error.
 int validate_bwd(const pith_attn_bwd_args* a, const char* who, bool need_dq, bool need_dkv);

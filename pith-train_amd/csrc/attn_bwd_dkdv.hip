@@ -422,6 +422,11 @@ int run_dkdv(const pith_attn_bwd_args* a, int split, void* workspace, hipStream_
     p.ws_dk = reinterpret_cast<float*>(workspace);
     p.ws_dv = p.ws_dk + (int64_t)split * a->B * a->Skv * a->Hkv * a->Dqk;
   }
+  // dS hand-over to the dQ call: only when the buffer is usable (otherwise the call behaves as without it)
+  if (a->ds && ds_bytes_for(a) > 0 && a->ds_bytes >= ds_bytes_for(a)) {
+    if ((uintptr_t)a->ds % 256) return fail(PITH_ERR_MISALIGNED, "%s: ds must be 256-byte aligned", who);
+    p.ds = reinterpret_cast<char*>(a->ds);
+  }
   if (a->Dqk == 128) launch_dkdv<128, 128>(p, a, st);
   else if (a->Dqk == 192) launch_dkdv<192, 128>(p, a, st);
   else launch_dkdv<64, 64>(p, a, st);

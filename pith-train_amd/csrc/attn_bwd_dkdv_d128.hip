@@ -48,7 +48,14 @@ struct TileCursor {
   }
 };
 
-template <bool CAUSAL, typename OutT>
+// EMIT_DS: wave B also stores every dS tile it forms (bf16, before the factor `scale`) to p.ds for
+// the dQ kernel of attn_bwd_dq_ds.hip, which then needs no score recomputation. Layout of p.ds:
+// one 4 KB image per (batch, query head, 64-row query tile, 128-key block, wave pair), in that
+// order; an image is the four bf16x8 fragments of the pair's B wave as they sit in registers,
+// 1 KB per 16-row step j, the 16 bytes of lane (g, c) at g*512 + ((c ^ 8g ^ 4(j&1)) << 4) (the
+// XOR terms make the reader's transposing LDS reads conflict-free). Keys at or beyond Skv hold 0
+// (their P is masked to 0).
+template <bool CAUSAL, typename OutT, bool EMIT_DS>
 __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams p) {
   constexpr int KS = kD / 16, DB = kD / 32;
   __shared__ __attribute__((aligned(1024))) char smem[kSmem];
@@ -207,7 +214,6 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(0);
   };
-
   // A: x = S of query tile mt -> P, left in the exchange buffer (fp32) and in frag (bf16).
   // Rows of the tile are queries q0 + 32*rb + acc_row(v, g); this lane's column is `key`.
   auto make_p = [&](const char* stage, int mt) __attribute__((always_inline)) {
@@ -222,14 +228,15 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) x[rb][v] = __builtin_amdgcn_exp2f(x[rb][v] * p.kappa - l4[rb][v >> 2][v & 3]);
-    if ((CAUSAL && q0 < kv_pair0 + 31) || (q0 + kBM > p.Sq)) {
-      // tile on the diagonal of a causal chunk, or a ragged last tile (wave-uniform branch)
+    if ((CAUSAL && q0 < kv_pair0 + 31) || (q0 + kBM > p.Sq) || (EMIT_DS && kv_pair0 + 32 > p.Skv)) {
+      // tile on the diagonal of a causal chunk, a ragged last tile, or (when dS is handed on, where
+      // nonexistent keys must read 0) the ragged last key block (wave-uniform branch)
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int qrow = q0 + 32 * rb + acc_row(v, g);
-          if ((CAUSAL && key > qrow) || qrow >= p.Sq) x[rb][v] = 0.f;
+          if ((CAUSAL && key > qrow) || qrow >= p.Sq || (EMIT_DS && key >= p.Skv)) x[rb][v] = 0.f;
         }
     }
 #pragma unroll
@@ -247,7 +254,14 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   };
   // B: x = dP of the tile in `stage`, P from the exchange buffer -> dS / scale in frag (bf16).
   // The factor `scale` of dS is applied once to the accumulated dK in the epilogue.
-  auto make_ds = [&](const char* stage) __attribute__((always_inline)) {
+  // `tile` is the (query head, tile) the stage holds (only used to place the dS image).
+  // With EMIT_DS the fragments are also stored as the image of query tile `tile` (layout at the top).
+  // The stores cost the kernel about 12 % wherever they are issued in the interval (measured: in this
+  // vector block, spread over B's matrix block, or at its end): each compute unit then has 16 KB of
+  // writes per interval in flight next to 33 KB of tile reads, its vector cache stalls on pending
+  // requests three times as often, and the sustained clock drops by 6 % under the write traffic.
+  char* const ds_wg = EMIT_DS ? p.ds + ((int64_t)n_tile * 4 + pair) * 4096 : nullptr;
+  auto make_ds = [&](const char* stage, const TileCursor& tile) __attribute__((always_inline)) {
     const float* delta_s = reinterpret_cast<const float*>(stage + 2 * kTile) + kBM;
     f32x4 pr[2][4], d4[2][4];
 #pragma unroll
@@ -266,6 +280,14 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
         frag[2 * rb + jj] = to_bf16x8(x[rb][8 * jj], x[rb][8 * jj + 1], x[rb][8 * jj + 2], x[rb][8 * jj + 3],
                                       x[rb][8 * jj + 4], x[rb][8 * jj + 5], x[rb][8 * jj + 6], x[rb][8 * jj + 7]);
     }
+    if constexpr (EMIT_DS) {
+      char* img = ds_wg + (((int64_t)(b * p.Hq + tile.hq) * p.ds_qt + tile.mt) * p.ds_kb) * (4 * 4096);
+      int off = (g << 9) + ((c ^ (g << 3)) << 4);  // recomputed per tile: no register is held across the interval
+      asm volatile("" : "+v"(off));
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        __builtin_nontemporal_store(frag[j], reinterpret_cast<bf16x8*>(img + j * 1024 + (off ^ ((j & 1) << 6))));
+    }
   };
 
   __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far: tile 0, stationary fragments
@@ -278,11 +300,15 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   // Ring stages rotate: prev <- cur <- next <- (the stage prev used to be).
   auto run = [&](auto role_tag) __attribute__((always_inline)) {
     constexpr bool ROLE_B = decltype(role_tag)::value;
-    TileCursor cur = {hq0, m_first};
+    TileCursor cur = {hq0, m_first}, done = cur;  // tiles i and i-1 of interval i
     int off_prev = 2 * kStage, off_cur = 0, off_next = kStage;
     auto end_interval = [&]() __attribute__((always_inline)) {
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // the tile requested in this interval has landed
+      // the tile requested in this interval has landed. Vector memory operations complete in issue
+      // order, and wave B issued its four dS stores after the request: they may stay in flight.
+      if (ROLE_B && EMIT_DS) __builtin_amdgcn_s_waitcnt(0x0F74);
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
+      done = cur;
       cur.advance(m_first, m_end);
       const int t = off_prev;
       off_prev = off_cur;
@@ -312,7 +338,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
         make_p(stage_cur, cur.mt);
       } else {
         if (will_request) request(smem + off_next);
-        make_ds(stage_prev);
+        make_ds(stage_prev, done);
         __syncthreads();
         matrix_block(stage_prev, stage_cur);
       }
@@ -323,7 +349,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
       transposed_product(smem + off_prev);
       __syncthreads();
     } else {
-      make_ds(smem + off_prev);
+      make_ds(smem + off_prev, done);
       __syncthreads();
       transposed_product(smem + off_prev);
     }
@@ -365,15 +391,21 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
 
 }  // namespace
 
-void launch_dkdv_d128(const BwdParams& p, bool causal, bool f32_out, unsigned grid, hipStream_t st) {
+template <bool EMIT_DS>
+static void launch_variant(const BwdParams& p, bool causal, bool f32_out, unsigned grid, hipStream_t st) {
   const dim3 g(grid), block(kThreads);
   if (causal) {
-    if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, float>), g, block, 0, st, p);
-    else hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, __bf16>), g, block, 0, st, p);
+    if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, float, EMIT_DS>), g, block, 0, st, p);
+    else hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, __bf16, EMIT_DS>), g, block, 0, st, p);
   } else {
-    if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<false, float>), g, block, 0, st, p);
-    else hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<false, __bf16>), g, block, 0, st, p);
+    if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<false, float, EMIT_DS>), g, block, 0, st, p);
+    else hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<false, __bf16, EMIT_DS>), g, block, 0, st, p);
   }
+}
+
+void launch_dkdv_d128(const BwdParams& p, bool causal, bool f32_out, unsigned grid, hipStream_t st) {
+  if (p.ds) launch_variant<true>(p, causal, f32_out, grid, st);
+  else launch_variant<false>(p, causal, f32_out, grid, st);
 }
 
 }  // namespace pith

@@ -290,12 +290,22 @@ BwdParams make_bwd_params(const pith_attn_bwd_args* a) {
   p.ws_dv = nullptr;
   p.k_pe = (const __bf16*)a->k_pe; p.k_pe_bs = a->k_pe_bs; p.k_pe_rs = a->k_pe_rs;
   p.ws_dkpe = nullptr;
+  p.ds = nullptr;
+  p.ds_qt = (int)((a->Sq + 63) / 64);
+  p.ds_kb = (int)((a->Skv + kDkdvBlockN - 1) / kDkdvBlockN);
   return p;
+}
+
+int64_t ds_bytes_for(const pith_attn_bwd_args* a) {
+  if (!a || a->Dqk != 128 || a->Dv != 128 || a->k_pe || a->B <= 0 || a->Hq <= 0 || a->Sq <= 0 || a->Skv <= 0) return 0;
+  return a->B * a->Hq * ((a->Sq + 63) / 64) * ((a->Skv + kDkdvBlockN - 1) / kDkdvBlockN) * (int64_t)(4 * 4096);
 }
 
 }  // namespace pith
 
 using namespace pith;
+
+extern "C" int64_t pith_attn_bwd_ds_bytes(const pith_attn_bwd_args* a) { return ds_bytes_for(a); }
 
 extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t stream) {
   const int rc = validate_bwd(a, "pith_attn_bwd_dq", true, false);
@@ -303,6 +313,16 @@ extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t strea
   const BwdParams p = make_bwd_params(a);
   hipStream_t st = (hipStream_t)stream;
   begin_launch();
+  if (a->ds && ds_bytes_for(a) > 0 && a->ds_bytes >= ds_bytes_for(a)) {
+    // dS was left by the dK/dV call of the same chunk: one product instead of three
+    if ((uintptr_t)a->ds % 256) return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_dq: ds must be 256-byte aligned");
+    BwdParams q = p;
+    q.ds = reinterpret_cast<char*>(a->ds);
+    q.tiles = (int)((a->Sq + 511) / 512);
+    q.accumulate = a->accumulate_dq;
+    launch_dq_from_ds(q, a->causal != 0, a->dq_dtype == PITH_F32, st);
+    return check_launch("pith_attn_bwd_dq");
+  }
   const bool half = a->Dqk == 192 || prefer_half_rows(a->Sq, a->Hq, a->B, a->causal != 0);
   if (a->Dqk == 192 || (a->Dqk == 128 && half)) {
     // early / late wave roles with 128-row workgroups whose wave pairs split every tile's keys: the

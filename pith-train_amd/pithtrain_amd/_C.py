@@ -81,6 +81,7 @@ class AttnBwdArgs(Structure):
         ("workspace", c_void_p), ("workspace_bytes", c_int64),
         ("k_pe", c_void_p), ("k_pe_bs", c_int64), ("k_pe_rs", c_int64),
         ("dk_pe", c_void_p), ("dk_pe_bs", c_int64),
+        ("ds", c_void_p), ("ds_bytes", c_int64),
     ]  # fmt: skip
 
 
@@ -125,6 +126,7 @@ SYMBOLS = {
     "pith_attn_bwd_dq": (c_int, [POINTER(AttnBwdArgs), c_void_p]),
     "pith_attn_bwd_dkdv_static": (c_int, [POINTER(AttnBwdArgs), c_void_p]),
     "pith_attn_bwd_dkdv_workspace_bytes": (c_int64, [POINTER(AttnBwdArgs)]),
+    "pith_attn_bwd_ds_bytes": (c_int64, [POINTER(AttnBwdArgs)]),
     "pith_cast_f32_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "pith_norm_rope_fwd": (c_int, [POINTER(NormRopeArgs), c_void_p]),
     "pith_norm_rope_bwd": (c_int, [POINTER(NormRopeArgs), c_void_p]),

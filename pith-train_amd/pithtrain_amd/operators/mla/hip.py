@@ -18,6 +18,7 @@ the underscore helpers allocate their outputs like the reference does.
 """
 
 import math
+import os
 
 import torch
 import torch.nn as nn
@@ -135,18 +136,68 @@ def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe=None) -> _C
         dq_bs=0, dk_bs=0, dv_bs=0, lse_bs=lse_bs, lse_hs=lse_hs,
         scale=float(softmax_scale), causal=int(bool(causal)),
         dq_dtype=_C.PITH_BF16, dkv_dtype=_C.PITH_BF16, accumulate_dq=0, accumulate_dkv=0,
-        workspace=None, workspace_bytes=0,
+        workspace=None, workspace_bytes=0, ds=None, ds_bytes=0,
     )  # fmt: skip
+
+
+def attn_bwd_ds_bytes(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> int:
+    """Bytes of the dS hand-over buffer for one chunk pair (0: these head dims have no hand-over path,
+    both backward calls then recompute the scores)."""
+    b, sq, hq, d_q = q.shape
+    args = _C.AttnBwdArgs(B=b, Sq=sq, Skv=k.shape[1], Hq=hq, Hkv=k.shape[2], Dqk=d_q, Dv=v.shape[-1])
+    return int(_C.lib().pith_attn_bwd_ds_bytes(_C.byref(args)))
+
+
+def _set_ds(args, ds: torch.Tensor, like: torch.Tensor) -> None:
+    if ds is None:
+        return
+    _C.require_device(like, ds)
+    assert ds.dtype == torch.uint8 and ds.is_contiguous() and ds.data_ptr() % 256 == 0, "ds must be a contiguous, 256-byte aligned uint8 buffer"
+    args.ds, args.ds_bytes = ds.data_ptr(), ds.numel()
+
+
+# Above this size the hand-over buffer is not worth its memory: the two backward calls recompute.
+# The hand-over makes the backward 3 % faster at the price of Sq*Skv*Hq*B*2 bytes of scratch (2 GiB per
+# ring step at 32 heads and 8192 x 4096 rows), so by default it is taken only while that stays small.
+DS_BUFFER_LIMIT_BYTES = int(float(os.environ.get("PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB", "1")) * (1 << 30))
+_DS_ROWS_PER_WORKGROUP = 512  # query rows a workgroup of the dS-reading dQ kernel owns
+_compute_units = {}
+
+
+def _device_compute_units(device: torch.device) -> int:
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx not in _compute_units:
+        info = _C.DeviceInfo()
+        _C.check(_C.lib().pith_device_info(idx, _C.byref(info)))
+        _compute_units[idx] = max(int(info.compute_units), 1)
+    return _compute_units[idx]
+
+
+def ds_buffer(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+    """A dS hand-over buffer for one chunk pair from torch's caching allocator, or None when the
+    shape has no hand-over path, the buffer would exceed DS_BUFFER_LIMIT_BYTES, or the dS-reading dQ
+    kernel would have fewer workgroups than the device has compute units (the recomputing kernels
+    use smaller workgroups and then win)."""
+    need = attn_bwd_ds_bytes(q, k, v)
+    if need == 0 or need > DS_BUFFER_LIMIT_BYTES:
+        return None
+    b, sq, hq, _ = q.shape
+    if -(-sq // _DS_ROWS_PER_WORKGROUP) * hq * b < _device_compute_units(q.device):
+        return None
+    return torch.empty(need, dtype=torch.uint8, device=q.device)
 
 
 def attn_bwd_dkdv_into(
     q, k, v, dout, lse, delta, dk: torch.Tensor, dv: torch.Tensor, softmax_scale: float, causal: bool,
-    accumulate: bool = False, k_pe: torch.Tensor = None, dk_pe: torch.Tensor = None,
+    accumulate: bool = False, k_pe: torch.Tensor = None, dk_pe: torch.Tensor = None, ds: torch.Tensor = None,
 ) -> None:  # fmt: skip
     """dk, dv <- (or +=, with accumulate) the gradients of this chunk pair; bf16 or fp32 outputs.
     With k_pe (see attn_fwd_into) dk is the gradient of k_nope and dk_pe [b, skv, 64] (contiguous rows,
-    same dtype as dk) receives the gradient of k_pe, summed over heads in head order."""
+    same dtype as dk) receives the gradient of k_pe, summed over heads in head order.
+    ds: uint8 buffer of attn_bwd_ds_bytes(q, k, v) bytes; the kernel leaves its dS tiles there for an
+    attn_bwd_dq_into call on the same chunk pair with the same buffer."""
     args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe)
+    _set_ds(args, ds, q)
     _C.require_device(q, dk, dv)
     assert dk.shape == k.shape and dv.shape == v.shape and dk.dtype == dv.dtype, "dk/dv must match k/v"
     if k_pe is not None:
@@ -173,10 +224,13 @@ def attn_bwd_dkdv_into(
 
 def attn_bwd_dq_into(
     q, k, v, dout, lse, delta, dq: torch.Tensor, softmax_scale: float, causal: bool, accumulate: bool = False,
-    k_pe: torch.Tensor = None,
+    k_pe: torch.Tensor = None, ds: torch.Tensor = None,
 ) -> None:  # fmt: skip
-    """dq <- (or +=, with accumulate) the query gradient of this chunk pair; bf16 or fp32 output."""
+    """dq <- (or +=, with accumulate) the query gradient of this chunk pair; bf16 or fp32 output.
+    ds: the buffer an attn_bwd_dkdv_into call on the same chunk pair has just filled; dq is then
+    computed from those dS tiles without recomputing the scores."""
     args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe)
+    _set_ds(args, ds, q)
     _C.require_device(q, dq)
     assert dq.shape == q.shape, "dq must match q"
     args.dq = dq.data_ptr()
@@ -258,8 +312,10 @@ def _attn_bwd_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Ten
                  causal: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:  # fmt: skip
     q, k, v, o, dout = q.contiguous(), k.contiguous(), v.contiguous(), o.contiguous(), dout.contiguous()
     delta = _mla_bwd_preprocess(o, dout)
-    dk, dv = _mla_bwd_dk_dv(q, k, v, dout, lse, delta, softmax_scale, causal)
-    dq = _mla_bwd_dq(q, k, v, dout, lse, delta, softmax_scale, causal)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    ds = ds_buffer(q, k, v)
+    attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, softmax_scale, causal, ds=ds)
+    attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, softmax_scale, causal, ds=ds)
     return dq, dk, dv
 
 

@@ -46,6 +46,7 @@ from pithtrain_amd.operators.mla.hip import (
     attn_bwd_dkdv_into,
     attn_bwd_dq_into,
     attn_fwd_into,
+    ds_buffer,
 )
 from pithtrain_amd.operators.ring_attention.combine import cast_f32_bf16_into, combine_into
 
@@ -252,12 +253,15 @@ class RingBackward:
         ks, vs = _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows)
         ls, dl = _lse_rows(self.lse, st.q_rows), _lse_rows(self.delta, st.q_rows)
         pes = _pe_rows(k_pe_j, st.kv_rows)
+        # The dK/dV kernel leaves its dS tiles in `hand` for the dQ kernel, which then skips the score
+        # recomputation (head dims 128/128; None otherwise: both kernels recompute).
+        hand = ds_buffer(qs, ks, vs) if pes is None else None
         attn_bwd_dkdv_into(qs, ks, vs, ds, ls, dl, _rows(dk_j, st.kv_rows), _rows(dv_j, st.kv_rows),
                            self.scale, st.causal, accumulate=add_to is not None, k_pe=pes,
-                           dk_pe=_pe_rows(dk_pe_j, st.kv_rows))  # fmt: skip
+                           dk_pe=_pe_rows(dk_pe_j, st.kv_rows), ds=hand)  # fmt: skip
         # Step 0 covers every row and initialises the accumulator; later steps add to their rows.
         attn_bwd_dq_into(qs, ks, vs, ds, ls, dl, _rows(self.dq_acc, st.q_rows), self.scale, st.causal,
-                         accumulate=self.done > 0, k_pe=pes)  # fmt: skip
+                         accumulate=self.done > 0, k_pe=pes, ds=hand)  # fmt: skip
         self.done += 1
         return (dk_j, dv_j) if k_pe_j is None else (dk_j, dv_j, dk_pe_j)
 

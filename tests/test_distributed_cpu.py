@@ -30,7 +30,7 @@ def _install_cpu_stand_ins():
     def attn_bwd_delta_into(out, dout, delta):
         delta.copy_(R.bwd_delta(out, dout))
 
-    def attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, scale, causal, accumulate=False, k_pe=None, dk_pe=None):
+    def attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, scale, causal, accumulate=False, k_pe=None, dk_pe=None, ds=None):
         _, rdk, rdv = R.chunk_bwd(q, full_key(k, k_pe), v, dout, lse.double(), delta.double(), scale, causal)
         if k_pe is not None:
             rpe, rdk = rdk[..., k.shape[-1] :].sum(2), rdk[..., : k.shape[-1]]
@@ -38,9 +38,12 @@ def _install_cpu_stand_ins():
         dk.copy_(dk.double() + rdk if accumulate else rdk)
         dv.copy_(dv.double() + rdv if accumulate else rdv)
 
-    def attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, scale, causal, accumulate=False, k_pe=None):
+    def attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, scale, causal, accumulate=False, k_pe=None, ds=None):
         rdq, _, _ = R.chunk_bwd(q, full_key(k, k_pe), v, dout, lse.double(), delta.double(), scale, causal)
         dq.copy_(dq.double() + rdq if accumulate else rdq)
+
+    def ds_buffer(q, k, v):  # no dS hand-over between the stand-ins
+        return None
 
     def combine_into(out1, lse1, out2, lse2, out, lse_out, base=0):
         o, l = R.combine_log2(out1.double(), lse1.double(), out2.double(), lse2.double())

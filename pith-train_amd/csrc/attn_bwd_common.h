@@ -67,6 +67,9 @@ constexpr int kDkdvBlockN = 128;
 // dK/dV for head dims (128, 128): attn_bwd_dkdv_d128.hip. p.tiles, p.split, p.ws_* are set by the caller.
 void launch_dkdv_d128(const BwdParams& p, bool causal, bool f32_out, unsigned grid, hipStream_t stream);
 
+// dK/dV for head dims (192, 128): attn_bwd_dkdv_d192.hip. Same conventions.
+void launch_dkdv_d192(const BwdParams& p, bool causal, bool f32_out, unsigned grid, hipStream_t stream);
+
 // dQ for head dims (128, 128): attn_bwd_dq_d128.hip. p.tiles = number of 256-row query tiles.
 void launch_dq_d128(const BwdParams& p, bool causal, bool f32_out, hipStream_t stream);
 

@@ -339,6 +339,8 @@ void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
   const bool f32 = a->dkv_dtype == PITH_F32;
   if constexpr (DQK == 128 && DV == 128) {
     launch_dkdv_d128(p, a->causal != 0, f32, grid.x, st);
+  } else if constexpr (DQK == 192 && DV == 128) {
+    launch_dkdv_d192(p, a->causal != 0, f32, grid.x, st);
   } else {
     if (a->causal) {
       if (f32) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DQK, DV, true, float>), grid, block, 0, st, p);

@@ -6,13 +6,23 @@
 // bound by the rate at which it can stream the images, not by the matrix pipe.
 //
 // Work split: a workgroup of 8 wavefronts owns 512 query rows of one (batch, head), wave w the 64-row
-// query tile 8*m_tile + w. Keys are visited in steps of 32 (one wave pair of the writer). Per step the
-// K tile (shared, packed and swizzled like everywhere else, 8 KB) and, per wave, the 4 KB image of its
-// tile for that pair (copied verbatim) go global -> LDS directly into a ring of four stages (160 KB),
-// requested three steps ahead (two steps in flight while one is in use): what bounds the kernel is how many bytes each compute unit keeps in
-// flight, so the stages are sized to spend the LDS on dS rather than on K. dQ^T += K^T dS^T: K^T
-// fragments come from transposing reads of the K tile and serve both 32-row blocks of the wave's
-// tile, dS^T fragments from transposing reads of the image, in the same key slot order.
+// query tile 8*m_tile + w of the writer. Keys are visited in steps of 32 (one wave pair of the
+// writer). Per step the K tile (shared, packed and swizzled like everywhere else, 8 KB) and, per
+// wave, the 4 KB image of its tile for that pair (copied verbatim) go global -> LDS directly. What
+// bounds the kernel is how many bytes of dS each compute unit keeps in flight (a compute unit's
+// vector cache holds about 64 outstanding 128-byte requests, i.e. ~8 KB per ~650 cycles of latency, so
+// every unit must stay busy and spend its requests on dS), so the LDS goes to dS: K tiles live in a
+// ring of 3 stages (they come from L2), the images in a ring of 4 stages of 32 KB. A wave's vector
+// loads complete in issue order, so one wave cannot wait for a K tile requested two steps ago without
+// also waiting for every image it requested before that tile; therefore waves 0..3 request the K
+// tiles and nothing else, and waves 4..7 request the images of all eight waves (each its own and that
+// of wave w - 4). Every wave waits for its own requests and the step's barrier publishes them.
+// dQ^T += K^T dS^T: K^T fragments come from transposing reads of the K tile and serve both 32-row
+// blocks of the wave's tile, dS^T fragments from transposing reads of the image, in the same key slot
+// order.
+// With 192-feature keys the same scheme was measured not to pay: a workgroup then holds accumulators
+// for 256 rows only, K is 43 % of the bytes a compute unit requests, and the kernel is no faster than
+// recomputing the scores.
 #include <type_traits>
 
 #include "attn_bwd_common.h"
@@ -21,29 +31,44 @@ namespace pith {
 namespace {
 
 constexpr int kThreads = 512;
-constexpr int kBM = 512;  // query rows per workgroup (64 per wave)
-constexpr int kBN = 32;   // keys per step
-constexpr int kD = 128;
-constexpr int kStages = 4;                       // power of two; steps s (in use), s+1 .. s+3 (in flight)
-constexpr int kKTile = kBN * kRowBytes128;       // 8 KB
-constexpr int kDsWave = 4096;                    // per wave and step
-constexpr int kStage = kKTile + 8 * kDsWave;     // 40 KB
-constexpr int kLoadsK = kBN * 16 / kThreads;     // K tile loads per wave and step (1)
-constexpr int kLoadsDs = 4;
+constexpr int kBN = 32;      // keys per step
+constexpr int kRingK = 3;    // K tiles: step s in use, s+1 and s+2 requested
 
-// s_waitcnt with vmcnt = n, the other counters left at their maxima (gfx9 encoding: vmcnt in bits
+// s_waitcnt with vmcnt = N, the other counters left at their maxima (gfx9 encoding: vmcnt in bits
 // 3:0 and 15:14).
 template <int N>
 __device__ __forceinline__ void wait_vector_loads_but() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
+// the same for a wave-uniform run-time count LO <= n <= HI, as a binary decision tree (a switch over
+// the counts compiles to a chain of one compare and branch per case, a few hundred cycles per call)
+template <int LO, int HI>
+__device__ __forceinline__ void wait_vector_loads_but(int n) {
+  if constexpr (LO == HI) {
+    wait_vector_loads_but<LO>();
+  } else {
+    constexpr int MID = (LO + HI) / 2;
+    if (n <= MID) wait_vector_loads_but<LO, MID>(n);
+    else wait_vector_loads_but<MID + 1, HI>(n);
+  }
+}
 
 template <bool CAUSAL, typename OutT>
 __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
-  constexpr int DB = kD / 32;
-  static_assert(kStages * kStage <= 160 * 1024, "the ring must fit the LDS");
-  __shared__ __attribute__((aligned(1024))) char smem[kStages * kStage];
+  constexpr int DQK = 128, DB = DQK / 32;
+  constexpr int QW = 64;                    // query rows per wave
+  constexpr int RBW = QW / 32;              // 32-row blocks per wave
+  constexpr int kBM = 8 * QW;               // query rows per workgroup
+  constexpr int kKStage = kBN * kRowBytes128;                        // 8 KB
+  constexpr int kDsWave = RBW * 2048;                                // per wave and step
+  constexpr int kDsStage = 8 * kDsWave;                              // 32 KB
+  constexpr int kRingD = 4;                                          // images: step s in use, the next three requested
+  constexpr int kOffDs = kRingK * kKStage;
+  constexpr int kLoadsDs = 2 * RBW;                                  // per image
+  constexpr int kLoadsK = 2;                                         // per K-moving wave and step
+  static_assert(kOffDs + kRingD * kDsStage <= 160 * 1024, "the rings must fit the LDS");
+  __shared__ __attribute__((aligned(1024))) char smem[kOffDs + kRingD * kDsStage];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -52,70 +77,98 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
   decode_block(blockIdx.x, p.Hq, p.B, p.tiles, m_tile, h, b);
   const int hk = h / p.group;
   const int m0 = m_tile * kBM;
-  const int mt = m_tile * 8 + wave;  // this wave's 64-row query tile
-  const int q_wave0 = mt * 64;
+  const int q_wave0 = m0 + wave * QW;
 
-  const int kv_row_bytes = p.Hkv * kD * 2;
-  const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * kD);
+  const int kv_row_bytes = p.Hkv * DQK * 2;
+  const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * DQK);
 
   // key steps: all of them, or up to the diagonal; a wave whose query tile does not exist (ragged
-  // Sq) has no images and visits nothing
+  // Sq) has no images and visits nothing. Rows q0 .. q0+QW-1 lie in the writer's 64-row tile q0 >> 6.
   const int n_steps_all = (p.Skv + kBN - 1) / kBN;
-  int n_steps_wg = n_steps_all, n_steps_wave = mt < p.ds_qt ? n_steps_all : 0;
-  if (CAUSAL) {
-    n_steps_wg = min(n_steps_all, (m0 + kBM - 1) / kBN + 1);
-    n_steps_wave = mt < p.ds_qt ? min(n_steps_all, (q_wave0 + 63) / kBN + 1) : 0;
-  }
+  const int n_steps_wg = CAUSAL ? min(n_steps_all, (m0 + kBM - 1) / kBN + 1) : n_steps_all;
+  auto steps_of = [&](int q0) __attribute__((always_inline)) {
+    if ((q0 >> 6) >= p.ds_qt) return 0;
+    return CAUSAL ? min(n_steps_all, (q0 + QW - 1) / kBN + 1) : n_steps_all;
+  };
+  const int n_steps_wave = steps_of(q_wave0);
+  // images of the query tile of rows q0..: key step s = pair s&3 of key block s>>2, 4 KB each,
+  // consecutive in s; the rows' part starts 1 KB per 16 rows into each image
+  auto images_of = [&](int q0) __attribute__((always_inline)) {
+    const int mt = min(q0 >> 6, p.ds_qt - 1);
+    return p.ds + (((int64_t)(b * p.Hq + h) * p.ds_qt + mt) * p.ds_kb) * (4 * 4096) + (q0 & 63) * 64;
+  };
 
-  // images of this wave's query tile: key step s = pair s&3 of key block s>>2, 4 KB each, consecutive in s
-  const char* ds_wave = p.ds + (((int64_t)(b * p.Hq + h) * p.ds_qt + (mt < p.ds_qt ? mt : 0)) * p.ds_kb) * (4 * 4096);
-
-  DirectTile128<kBN, kThreads> mover;
-  mover.init(kv_row_bytes, wave, lane);
-  auto request = [&](int s) __attribute__((always_inline)) {
-    char* stage = smem + (s & (kStages - 1)) * kStage;
-    mover.issue(kh + (int64_t)s * kBN * kv_row_bytes, p.Skv - s * kBN, stage, wave, lane);
-    if (s < n_steps_wave) {
-      const char* src = ds_wave + (int64_t)s * 4096;
-      char* dst = stage + kKTile + wave * kDsWave;
-      int off = lane << 4;
-      asm volatile("" : "+v"(off));
+  // ---- requests. Waves 0..3: K tiles. Waves 4..7: the dS parts of waves w-4 and w.
+  const bool k_mover = wave < 4;
+  DirectTile128<kBN, 256> mover;
+  mover.init(kv_row_bytes, wave & 3, lane);
+  const char* ds_src[2] = {images_of(q_wave0 - 4 * QW), images_of(q_wave0)};        // only used by waves 4..7
+  const int ds_steps[2] = {k_mover ? 0 : steps_of(q_wave0 - 4 * QW), k_mover ? 0 : n_steps_wave};
+  auto request_k = [&](int s, int slot) __attribute__((always_inline)) {
+    char* stage = smem + slot * kKStage;
+    const char* k_src = kh + (int64_t)s * kBN * kv_row_bytes;
+    mover.issue(k_src, p.Skv - s * kBN, stage, wave & 3, lane);
+  };
+  auto request_ds = [&](int s, int slot) __attribute__((always_inline)) {
+    int off = lane << 4;
+    asm volatile("" : "+v"(off));
 #pragma unroll
-      for (int j = 0; j < 4; ++j) load_lds16(src + j * 1024, off, dst + j * 1024);
-    }
+    for (int r = 0; r < 2; ++r)
+      if (s < ds_steps[r]) {
+        const char* src = ds_src[r] + (int64_t)s * 4096;
+        char* dst = smem + kOffDs + slot * kDsStage + (wave - 4 + 4 * r) * kDsWave;
+#pragma unroll
+        for (int j = 0; j < kLoadsDs; ++j) load_lds16(src + j * 1024, off, dst + j * 1024);
+      }
   };
   // loads this wave issued for step t
-  auto loads_of = [&](int t) __attribute__((always_inline)) { return t >= n_steps_wg ? 0 : (t < n_steps_wave ? kLoadsK + kLoadsDs : kLoadsK); };
-  // waits until this wave's loads for step s have landed. At that point steps s+1 .. s+kStages-2 have
-  // been requested as well (step s+kStages-1 follows after the barrier) and may stay in flight.
+  auto loads_of = [&](int t) __attribute__((always_inline)) {
+    if (t >= n_steps_wg) return 0;
+    if (k_mover) return kLoadsK;
+    return (t < ds_steps[0] ? kLoadsDs : 0) + (t < ds_steps[1] ? kLoadsDs : 0);
+  };
+  // ring slots of step s (K tiles, dS parts) and of the steps to request next; advanced by one per step
+  int k_slot = 0, k_next = kRingK - 1, d_slot = 0, d_next = kRingD - 1;
+  auto advance = [&]() __attribute__((always_inline)) {
+    k_slot = k_slot + 1 == kRingK ? 0 : k_slot + 1;
+    k_next = k_next + 1 == kRingK ? 0 : k_next + 1;
+    d_slot = d_slot + 1 == kRingD ? 0 : d_slot + 1;
+    d_next = d_next + 1 == kRingD ? 0 : d_next + 1;
+  };
+  // waits until this wave's loads for step s have landed: the steps requested after it (all but the
+  // last of the ring, which follows after the barrier) may stay in flight. Away from the end of the key
+  // range that is a constant number of loads.
+  constexpr int kSteadyDs = (kRingD - 2) * 2 * kLoadsDs;
+  static_assert(kRingK == 3 && kSteadyDs < 32, "one K step in flight; dS loads in flight fit the decision tree");
+  const int ds_steady_end = min(min(ds_steps[0], ds_steps[1]), n_steps_wg) - (kRingD - 2);  // steps below: steady state
   auto wait_step = [&](int s) __attribute__((always_inline)) {
-    static_assert(kStages == 4, "the list of counts below is for two steps in flight");
-    const int n = loads_of(s + 1) + loads_of(s + 2);  // one of 0, 1, 2, 5, 6, 10
-    if (n >= 10) wait_vector_loads_but<10>();
-    else if (n >= 6) wait_vector_loads_but<6>();
-    else if (n >= 5) wait_vector_loads_but<5>();
-    else if (n >= 2) wait_vector_loads_but<2>();
-    else if (n >= 1) wait_vector_loads_but<1>();
-    else wait_vector_loads_but<0>();
+    if (k_mover) {
+      if (s + 1 < n_steps_wg) wait_vector_loads_but<kLoadsK>();
+      else wait_vector_loads_but<0>();
+    } else if (s < ds_steady_end) {
+      wait_vector_loads_but<kSteadyDs>();
+    } else {
+      int n = 0;
+#pragma unroll
+      for (int d = 1; d < kRingD - 1; ++d) n += loads_of(s + d);
+      wait_vector_loads_but<0, 31>(n);
+    }
   };
 
-  f32x16 acc[2][DB];  // [32-row block of the tile][feature block]
+  f32x16 acc[RBW][DB];  // [32-row block][feature block]
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb)
+  for (int rb = 0; rb < RBW; ++rb)
 #pragma unroll
     for (int o = 0; o < DB; ++o)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[rb][o][v] = 0.f;
 
-  // per-lane read offsets. K tile: transposing reads of feature block o, lower / upper 8 keys of a
-  // 16-key step. Image: this lane supplies, for its 16-lane block (g, chalf) and r = 4i + m, the 8
-  // bytes that hold key 4g + i (+ 8 for the upper read) at queries 16*chalf + 4m .. +3 of a 32-row
-  // block: 16-row step chalf of the block, writer lane group m&1, fragment half m>>1.
-  int t_off[DB][2];
-#pragma unroll
-  for (int o = 0; o < DB; ++o)
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) t_off[o][hh] = transposed_offset128(0, hh, 32 * o, lane);
+  // per-lane read offsets. K tile: transposing reads of the lower / upper 8 keys of a 16-key step at
+  // feature block 0; block o follows by XOR with o << 6 (the swizzle is an XOR of the piece index).
+  // Image: this lane supplies, for its 16-lane block (g, chalf) and r = 4i + m, the 8 bytes that hold
+  // key 4g + i (+ 8 for the upper read) at queries 16*chalf + 4m .. +3 of a 32-row block: 16-row step
+  // chalf of the block, writer lane group m&1, fragment half m>>1.
+  const int t_base[2] = {transposed_offset128(0, 0, 0, lane), transposed_offset128(0, 1, 0, lane)};
   int ds_off[2];
   {
     const int r = lane & 15, chalf = (lane >> 4) & 1;
@@ -125,46 +178,57 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
     ds_off[1] = ds_off[0] ^ 128;  // key + 8: bit 3 of the key index
   }
 
-  auto compute = [&](const char* stage) __attribute__((always_inline)) {
-    const char* img = stage + kKTile + wave * kDsWave;
+  auto compute = [&](const char* stage, const char* img) __attribute__((always_inline)) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {  // 16 keys each
-      bf16x8 dsf[2];
+      bf16x8 dsf[RBW];
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
+      for (int rb = 0; rb < RBW; ++rb) {
         const char* d = img + rb * 2048 + ks * 256;
         dsf[rb] = lds_read_transposed_at(d + ds_off[0], d + ds_off[1]);
       }
-      const char* kt = stage + ks * 16 * kRowBytes128;
 #pragma unroll
       for (int o = 0; o < DB; ++o) {
-        const bf16x8 a = lds_read_transposed_at(kt + t_off[o][0], kt + t_off[o][1]);
+        const char* kt = stage + ks * 16 * kRowBytes128;
+        const bf16x8 a = lds_read_transposed_at(kt + (t_base[0] ^ (o << 6)), kt + (t_base[1] ^ (o << 6)));
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb) acc[rb][o] = mfma32(a, dsf[rb], acc[rb][o]);
+        for (int rb = 0; rb < RBW; ++rb) acc[rb][o] = mfma32(a, dsf[rb], acc[rb][o]);
       }
     }
   };
 
+  if (k_mover) {
 #pragma unroll
-  for (int d = 0; d < kStages - 1; ++d)
-    if (d < n_steps_wg) request(d);
+    for (int d = 0; d < kRingK - 1; ++d)
+      if (d < n_steps_wg) request_k(d, d);
+  } else {
+#pragma unroll
+    for (int d = 0; d < kRingD - 1; ++d)
+      if (d < n_steps_wg) request_ds(d, d);
+  }
   auto step = [&](int s, auto compute_tag) __attribute__((always_inline)) {
     wait_step(s);
-    __syncthreads();  // every wave's part of step s has landed; everyone is done with step s-1
-    if (s + kStages - 1 < n_steps_wg) request(s + kStages - 1);
-    if constexpr (decltype(compute_tag)::value) compute(smem + (s & (kStages - 1)) * kStage);
+    __syncthreads();  // every wave's requests for step s have landed; everyone is done with step s-1
+    if (k_mover) {
+      if (s + kRingK - 1 < n_steps_wg) request_k(s + kRingK - 1, k_next);
+    } else {
+      if (s + kRingD - 1 < n_steps_wg) request_ds(s + kRingD - 1, d_next);
+    }
+    if constexpr (decltype(compute_tag)::value)
+      compute(smem + k_slot * kKStage, smem + kOffDs + d_slot * kDsStage + wave * kDsWave);
+    advance();
   };
   int s = 0;
   for (; s < n_steps_wave; ++s) step(s, std::true_type{});
-  // other waves of the workgroup may still have steps to visit: keep moving K tiles, keep in step
+  // other waves of the workgroup may still have steps to visit: keep moving tiles, keep in step
   for (; s < n_steps_wg; ++s) step(s, std::false_type{});
 
-  OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * kD;
+  OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * DQK;
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < RBW; ++rb) {
     const int qrow = q_wave0 + 32 * rb + c;
     if (qrow < p.Sq) {
-      OutT* dst = dqh + qrow * ((int64_t)p.Hq * kD);
+      OutT* dst = dqh + qrow * ((int64_t)p.Hq * DQK);
 #pragma unroll
       for (int o = 0; o < DB; ++o)
 #pragma unroll

@@ -18,7 +18,7 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpith_hip.so")
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 
-SOURCES = ["api.hip", "combine.hip", "norm_rope.hip", "mla_assemble.hip", "attn_fwd.hip", "attn_fwd_direct.hip", "attn_bwd_dq.hip", "attn_bwd_dq_d128.hip", "attn_bwd_dq_direct.hip", "attn_bwd_dq_ds.hip", "attn_bwd_dkdv.hip", "attn_bwd_dkdv_d128.hip"]
+SOURCES = ["api.hip", "combine.hip", "norm_rope.hip", "mla_assemble.hip", "attn_fwd.hip", "attn_fwd_direct.hip", "attn_bwd_dq.hip", "attn_bwd_dq_d128.hip", "attn_bwd_dq_direct.hip", "attn_bwd_dq_ds.hip", "attn_bwd_dkdv.hip", "attn_bwd_dkdv_d128.hip", "attn_bwd_dkdv_d192.hip"]
 
 # -packed-fp32-ops is switched off on purpose: some packed fp32 forms have produced wrong results
 # on the target machines. Code object v5 is understood by both the ROCm 7.0 runtime bundled with

@@ -33,18 +33,18 @@ SHAPES = [
 NONCAUSAL_SHAPES = SHAPES + [(1, 512, 256, 8, 2), (1, 256, 768, 4, 4), (1, 200, 450, 4, 2), (1, 65, 129, 2, 2)]
 
 
-def _inputs(B, Sq, Skv, Hq, Hkv, seed=42):
+def _inputs(B, Sq, Skv, Hq, Hkv, seed=42, dqk=128):
     g = torch.Generator().manual_seed(seed)
-    scale = 128**-0.5
-    q = (torch.randn(B, Sq, Hq, 128, generator=g) * scale).to(torch.bfloat16)
-    k = (torch.randn(B, Skv, Hkv, 128, generator=g) * scale).to(torch.bfloat16)
+    scale = dqk**-0.5
+    q = (torch.randn(B, Sq, Hq, dqk, generator=g) * scale).to(torch.bfloat16)
+    k = (torch.randn(B, Skv, Hkv, dqk, generator=g) * scale).to(torch.bfloat16)
     v = (torch.randn(B, Skv, Hkv, 128, generator=g) * scale).to(torch.bfloat16)
     dout = torch.randn(B, Sq, Hq, 128, generator=g).to(torch.bfloat16)
     return q, k, v, dout, scale
 
 
-def _run(gpu, causal, shape, dq_dtype):
-    q, k, v, dout, scale = _inputs(*shape)
+def _run(gpu, causal, shape, dq_dtype, dqk=128):
+    q, k, v, dout, scale = _inputs(*shape, dqk=dqk)
     qd, kd, vd, dod = (t.to(gpu) for t in (q, k, v, dout))
     o, lse = _mla_fwd(qd, kd, vd, scale, causal)
     delta = _mla_bwd_preprocess(o, dod)
@@ -100,8 +100,10 @@ def test_small_buffer_falls_back_to_recomputation(gpu):
     attn_bwd_dq_into(qd, kd, vd, dod, lse, delta, dq1, scale, True, ds=small)
     assert torch.equal(dq0, dq1)
     # head dims without a hand-over path report 0 bytes and get no buffer
-    q192 = torch.empty(1, 128, 4, 192, dtype=torch.bfloat16, device=gpu)
-    assert attn_bwd_ds_bytes(q192, q192, qd[:, :128]) == 0 and ds_buffer(q192, q192, qd[:, :128]) is None
+    for d in (64, 192):
+        qx = torch.empty(1, 128, 4, d, dtype=torch.bfloat16, device=gpu)
+        vx = torch.empty(1, 128, 4, min(d, 128), dtype=torch.bfloat16, device=gpu)
+        assert attn_bwd_ds_bytes(qx, qx, vx) == 0 and ds_buffer(qx, qx, vx) is None
 
 
 @pytest.mark.parametrize("layout", ["contiguous", "zigzag"])

@@ -410,6 +410,8 @@ def main():
                     help="skip the MLA 16K and long 131K configurations (sub-objects mla16k, long131k)")
     ap.add_argument("--config", choices=["mla16k", "long131k"], default=None,
                     help="time only this configuration's ring share and print its sub-object (for kernel traces)")
+    ap.add_argument("--handover", action="store_true",
+                    help="run the headline share with the dS hand-over between the backward kernels switched on (for traces)")
     ap.add_argument("--counter-pass", action="store_true",
                     help="run only the roofline kernel and a calibration copy (for rocprofv3 --pmc), print no JSON")
     args = ap.parse_args()
@@ -425,6 +427,10 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.handover:
+        from pithtrain_amd.operators.mla import hip
+
+        hip.DS_BUFFER_LIMIT_BYTES = 1 << 40
     if args.config:
         cfg = MLA16K if args.config == "mla16k" else LONG131K
         print(json.dumps({args.config: bench_other_config(torch, device, cfg, args.steps, args.warmup)}))

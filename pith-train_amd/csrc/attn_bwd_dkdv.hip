@@ -1,4 +1,6 @@
-// Key/value-gradient kernel of one chunk attention backward for gfx950, against an external
+// Key/value-gradient kernel of one chunk attention backward for gfx950 with register-staged tiles
+// (used for head dims 64/64; 128/128 and 192/128 have direct-load kernels of their own), the entry
+// points of the dK/dV step and the reduction kernel of the head split; against an external
 // (ring-combined) base-2 LSE and delta = rowsum(O*dO). Follows
 // pithtrain/operators/mla/triton.py:130-197 (non-causal :331-384): P = exp2(kappa*s - lse2) in
 // fp32, masked entries 0, P rounded to bf16 for dV += P^T dO, dS = P*(dP - delta)*scale rounded
@@ -12,7 +14,7 @@
 //     wave B:  dP = dO V^T ->  dS = P o (dP - delta) * scale -> dK^T += Q^T dS (holds V, dK)
 // B needs A's P: A leaves the fp32 P tile (32 x 32) in an LDS exchange buffer, in the lane order
 // both waves share, and B picks it up after the iteration's only barrier. Both waves issue the
-// same number of MFMAs (also for 192/128 head dims: 12 + 8 against 8 + 12).
+// same number of MFMAs.
 // The stationary side (K or V rows) sits in registers as B operands, so score tiles have the key
 // index as their column; P / dS then feed the products that contract over queries straight from
 // registers (slot order, see attn_tiles.h) with dO^T / Q^T read transposed from LDS.
@@ -171,10 +173,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
 
   const int64_t q_row_stride = (int64_t)p.Hq * DQK;
   const int64_t do_row_stride = (int64_t)p.Hq * DV;
-  // keys in two parts (192-feature keys only): k and dk rows hold 128 features per head, the last 64
-  // features come from k_pe (one vector per position) and their gradient goes, per head, to ws_dkpe
-  const bool two_part = DQK == 192 && p.k_pe != nullptr;
-  const int k_head = two_part ? 128 : DQK;
+  const int k_head = DQK;
   const int64_t k_row_stride = (int64_t)p.Hkv * k_head;
   const int64_t v_row_stride = (int64_t)p.Hkv * DV;
 
@@ -184,10 +183,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
     const int row = key < p.Skv ? key : p.Skv - 1;
     if (!role_b) {
       const __bf16* src = p.k + b * p.k_bs + row * k_row_stride + (int64_t)hk * k_head + g * 8;
-      const __bf16* src_pe = two_part ? p.k_pe + b * p.k_pe_bs + row * p.k_pe_rs + g * 8 : src + 128;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        stat[ks] = *reinterpret_cast<const bf16x8*>(ks < 8 ? src + ks * 16 : src_pe + (ks - 8) * 16);
+      for (int ks = 0; ks < KS; ++ks) stat[ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
     } else {
       const __bf16* src = p.v + b * p.v_bs + row * v_row_stride + (int64_t)hk * DV + g * 8;
 #pragma unroll
@@ -250,16 +247,6 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
     const int d = role_b ? k_head : DV;
     const int nblk = role_b ? k_head / 32 : DVB;
     const int64_t row_stride = role_b ? k_row_stride : v_row_stride;
-    if (two_part && role_b) {  // this head's gradient of the shared rotary part: [Hkv][B][Skv][64] fp32
-      float* ws = p.ws_dkpe + (((int64_t)hk * p.B + b) * p.Skv + key) * 64;
-#pragma unroll
-      for (int o = 4; o < NACC; ++o)
-        if (o < DB)
-#pragma unroll
-          for (int b4 = 0; b4 < 4; ++b4)
-            store4<float>(ws + 32 * (o - 4) + 8 * b4 + 4 * g, acc[o][4 * b4], acc[o][4 * b4 + 1], acc[o][4 * b4 + 2],
-                          acc[o][4 * b4 + 3], false);
-    }
     if (p.split > 1) {
       float* ws = (role_b ? p.ws_dk : p.ws_dv) +
                   (((int64_t)part * p.B + b) * p.Skv + key) * row_stride + (int64_t)hk * d;

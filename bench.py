@@ -54,10 +54,12 @@ FROM_PROFILES = {
     "note": "quoted from committed rocprofv3 summaries, not measured in this run",
     "attn_bwd_dkdv_d128_kernel<non-causal>": {
         "file": "profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt",
-        "hbm_bytes_per_launch": 282_700_000,  # 215.6 MB fetched + 67.1 MB written (FETCH_SIZE / WRITE_SIZE, calibrated on a copy)
+        # with the dS stores: 215.6 MB fetched + 2281.7 MB written (2147.5 MB of dS, 67.1 MB of head-split partials...)
+        "hbm_bytes_per_launch": 2_430_000_000,
+        "hbm_bytes_per_launch_without_ds_stores": 282_700_000,  # 215.6 MB fetched + 67.1 MB written
         "mfma_file": "profiles/attn_kernels_mfma_lds_counters.txt",
-        "mfma_busy_fraction": 0.615,  # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs)
-        "sustained_clock_ghz": 1.85,  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration (2.4 GHz nominal)
+        "mfma_busy_fraction": 0.54,  # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs); 0.615 without the stores
+        "sustained_clock_ghz": 1.75,  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration (2.4 GHz nominal); 1.85 without the stores
     },
     "combine_front_kernel": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_per_launch": COMBINE_TRAFFIC},
     "norm_rope_kernels": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_fwd_plus_bwd": 159_400_000 + 235_200_000},
@@ -152,25 +154,23 @@ def ring_summary(cfg, ms_step, ms_fwd, ms_bwd):
     }  # fmt: skip
 
 
-def bench_handover(torch, dev_inputs, steps, warmup):
-    """The headline share once more with the dS hand-over between the two backward kernels switched on
-    for every step (by default it is declined above 1 GiB of scratch, which this share exceeds)."""
+def bench_recompute(torch, dev_inputs, steps, warmup):
+    """The headline share once more with the dS hand-over between the two backward kernels switched off:
+    both kernels recompute S and dP (7 matrix products executed for the 5 counted), no scratch."""
     from pithtrain_amd.operators.mla import hip
 
     limit = hip.DS_BUFFER_LIMIT_BYTES
-    hip.DS_BUFFER_LIMIT_BYTES = 1 << 40
+    hip.DS_BUFFER_LIMIT_BYTES = 0
     try:
         ms_step, ms_fwd, ms_bwd, _, _ = time_ring_share(torch, QWEN3, dev_inputs, steps, warmup)
     finally:
         hip.DS_BUFFER_LIMIT_BYTES = limit
     fwd_flops, bwd_flops = QWEN3.flops()
-    q, ks = dev_inputs[0], dev_inputs[1]
-    scratch = q.shape[2] * q.shape[1] * (ks[0].shape[1] // 2) * 2
     return {
-        "what": "the same share with the dK/dV kernel handing its dS tiles to the dQ kernel (5 matrix products instead of 7; "
-                "PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB >= 2)",
+        "what": "the same share with the dS hand-over off (PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB=0): dQ and dK/dV kernels both "
+                "recompute S and dP",
         "ms_per_step": round(ms_step, 4), "tflops": round((fwd_flops + bwd_flops) / (ms_step * 1e-3) / 1e12, 2),
-        "bwd_ms": round(ms_bwd, 4), "scratch_bytes_per_ring_step": int(scratch),
+        "bwd_ms": round(ms_bwd, 4),
     }  # fmt: skip
 
 
@@ -183,7 +183,7 @@ def bench_other_config(torch, device, cfg, steps, warmup):
 
 
 def bench_ring(torch, args, dev_inputs):
-    from pithtrain_amd.operators.mla.hip import attn_bwd_delta_into, attn_bwd_dkdv_into
+    from pithtrain_amd.operators.mla.hip import attn_bwd_delta_into, attn_bwd_dkdv_into, ds_buffer
     from pithtrain_amd.operators.ring_attention.local import ring_schedule
 
     q, ks, vs, dout = dev_inputs
@@ -201,10 +201,12 @@ def bench_ring(torch, args, dev_inputs):
         rows = slice(s.q_rows[0], s.q_rows[1])
         dk, dv = torch.empty_like(k_j), torch.empty_like(v_j)
         launches.append((q[:, rows], k_j, v_j, dout[:, rows], lse[:, :, rows], delta[:, :, rows], dk, dv))
+    # the same kernel variant as in the step: with the dS hand-over buffer whenever the ring driver would use one
+    hand = ds_buffer(*launches[0][:3])
 
     def dkdv_launches():
         for a in launches:
-            attn_bwd_dkdv_into(*a, scale, False)
+            attn_bwd_dkdv_into(*a, scale, False, ds=hand)
 
     dkdv_launches()
     if args.counter_pass:
@@ -220,7 +222,7 @@ def bench_ring(torch, args, dev_inputs):
     ms_dkdv = time_events(torch, dkdv_launches, args.steps) / len(launches)
     entries = (S_LOCAL * S_LOCAL // 2) * HQ
     dkdv_flops = 2 * (2 * DQK + 2 * DV) * entries
-    return ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops
+    return ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops, hand is not None
 
 
 def bench_combine(torch, device, reps=50, graph=True):
@@ -410,8 +412,8 @@ def main():
                     help="skip the MLA 16K and long 131K configurations (sub-objects mla16k, long131k)")
     ap.add_argument("--config", choices=["mla16k", "long131k"], default=None,
                     help="time only this configuration's ring share and print its sub-object (for kernel traces)")
-    ap.add_argument("--handover", action="store_true",
-                    help="run the headline share with the dS hand-over between the backward kernels switched on (for traces)")
+    ap.add_argument("--no-handover", action="store_true",
+                    help="run everything with the dS hand-over between the backward kernels switched off (for traces)")
     ap.add_argument("--counter-pass", action="store_true",
                     help="run only the roofline kernel and a calibration copy (for rocprofv3 --pmc), print no JSON")
     args = ap.parse_args()
@@ -427,10 +429,10 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    if args.handover:
+    if args.no_handover:
         from pithtrain_amd.operators.mla import hip
 
-        hip.DS_BUFFER_LIMIT_BYTES = 1 << 40
+        hip.DS_BUFFER_LIMIT_BYTES = 0
     if args.config:
         cfg = MLA16K if args.config == "mla16k" else LONG131K
         print(json.dumps({args.config: bench_other_config(torch, device, cfg, args.steps, args.warmup)}))
@@ -446,10 +448,10 @@ def main():
         bench_mla_assemble(torch, device, reps=3)
         print("counter pass done")
         return
-    ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops = ring
-    handover = None
-    if not args.no_extra_configs:
-        handover = bench_handover(torch, dev_inputs, args.steps, args.warmup)
+    ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops, handover_on = ring
+    recompute = None
+    if not args.no_extra_configs and handover_on:
+        recompute = bench_recompute(torch, dev_inputs, args.steps, args.warmup)
     del dev_inputs
     torch.cuda.empty_cache()
     fwd_flops, bwd_flops = flops_per_step()
@@ -514,13 +516,20 @@ def main():
             "frac_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         },
         "roofline": {
-            "kernel": "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step)",
+            "kernel": "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step"
+                      + ("; also stores its dS tiles for the dQ kernel)" if handover_on else ")"),
             "bound": "mfma", "achieved": round(dkdv_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": dkdv_prof["hbm_bytes_per_launch"], "traffic_from": dkdv_prof["file"],
+            "traffic": dkdv_prof["hbm_bytes_per_launch" if handover_on else "hbm_bytes_per_launch_without_ds_stores"],
+            "traffic_from": dkdv_prof["file"],
             "ms_per_launch": round(ms_dkdv, 4),
         },  # fmt: skip
-        "ds_handover": handover,
+        "ds_handover": {
+            "on": handover_on,
+            "what": "the dK/dV kernel hands its dS tiles to the dQ kernel (5 matrix products executed instead of 7)",
+            "scratch_bytes_per_ring_step": HQ * S_LOCAL * (S_LOCAL // 2) * 2 if handover_on else 0,
+            "recompute_backward": recompute,
+        },
         "mla16k": mla16k,
         "long131k": long131k,
         "combine": {

@@ -302,7 +302,9 @@ int pick_split(const pith_attn_bwd_args* a) {
   const int64_t group = a->Hq / a->Hkv;
   const int64_t base = ((a->Skv + kBN - 1) / kBN) * a->Hkv * a->B;
   int split = 1;
-  const int64_t want = 2 * (int64_t)compute_units_or_default();  // two rounds of workgroups
+  // one workgroup per compute unit is resident; without a causal mask all workgroups carry the same
+  // work, so one full round is ideal; under the mask two rounds (heaviest first) balance better
+  const int64_t want = (a->causal ? 2 : 1) * (int64_t)compute_units_or_default();
   while (split < group && base * split < want && group % (split * 2) == 0) split *= 2;
   return split;
 }

@@ -87,11 +87,12 @@ def test_static_scratch_entry_causal_and_accumulate(gpu):
 
 def test_static_scratch_entry_rejects_what_does_not_fit(gpu):
     lib = _C.lib()
-    # 48 key tiles of 4 kv heads are cut 4 ways over their 4 query heads: the partial sums need
-    # 4 x 6144 x 4 x 256 x 4 bytes = 96 MiB > the 64 MiB scratch. Nothing is launched.
-    B, Sq, Skv, Hq, Hkv, D = 1, 64, 6144, 16, 4, 128
+    # a causal call: 48 key tiles of 4 kv heads are cut 4 ways over their 4 query heads (two rounds of
+    # workgroups on 256 compute units): the partial sums need 4 x 6144 x 4 x 256 x 4 bytes = 96 MiB > the
+    # 64 MiB scratch. Nothing is launched.
+    B, Sq, Skv, Hq, Hkv, D = 1, 6144, 6144, 16, 4, 128
     q, k, v, dout, lse, delta, scale = _inputs(gpu, 3, B, Sq, Skv, Hq, Hkv, D)
-    args = _bwd_args(q, k, v, dout, lse, delta, scale, False)
+    args = _bwd_args(q, k, v, dout, lse, delta, scale, True)
     need = lib.pith_attn_bwd_dkdv_workspace_bytes(ctypes.byref(args))
     assert need > 64 << 20
     dk, dv = torch.empty_like(k), torch.empty_like(v)

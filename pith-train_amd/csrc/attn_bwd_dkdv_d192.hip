@@ -164,6 +164,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
       const __bf16* src = p.v + b * p.v_bs + row * v_row_stride + (int64_t)hk * kDV + g * 8;
 #pragma unroll
       for (int ks = 0; ks < VS; ++ks) stat[ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
+      // wave B works with -V: its score-type product then starts from delta and yields delta - dP,
+      // i.e. -(dP - delta) without a subtraction per element; the factor -scale on the accumulated dK
+      // undoes the sign
+#pragma unroll
+      for (int ks = 0; ks < VS; ++ks) stat[ks] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, stat[ks]) ^ 0x80008000u);
     }
   }
   f32x16 acc[DB];  // A uses the first DVB of them
@@ -211,12 +216,28 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
     }
   };
 
+  // x starts from 0 in wave A and from the delta values of the tile's rows in wave B
+  auto start_x = [&](const char* stage, auto role_tag) __attribute__((always_inline)) {
+    if constexpr (decltype(role_tag)::value) {
+      const float* delta_s = reinterpret_cast<const float*>(stage + kOffStat) + kBM;
+#pragma unroll
+      for (int rb = 0; rb < TB; ++rb)
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          const f32x4 d = *reinterpret_cast<const f32x4*>(delta_s + 32 * rb + 8 * b4 + 4 * g);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) x[rb][4 * b4 + e] = d[e];
+        }
+    } else {
+#pragma unroll
+      for (int rb = 0; rb < TB; ++rb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[rb][v] = 0.f;
+    }
+  };
   auto straight_product = [&](const char* stage, auto role_tag) __attribute__((always_inline)) {
     constexpr int NS = decltype(role_tag)::value ? VS : KS;
-#pragma unroll
-    for (int rb = 0; rb < TB; ++rb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) x[rb][v] = 0.f;
+    start_x(stage, role_tag);
 #pragma unroll
     for (int ks = 0; ks < NS; ++ks)
 #pragma unroll
@@ -241,6 +262,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
     for (int j = 0; j < 2 * TB; ++j)
 #pragma unroll
       for (int o = 0; o < NO; ++o) at[j][o] = transposed_frag(stage_prev, j, o, role_tag);
+    start_x(stage_cur, role_tag);
 #pragma unroll
     for (int ks = 0; ks < NS0; ++ks)
 #pragma unroll
@@ -249,10 +271,6 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
     for (int j = 0; j < 2 * TB; ++j)
 #pragma unroll
       for (int o = 0; o < NO; ++o) acc[o] = mfma32(at[j][o], frag[j], acc[o]);
-#pragma unroll
-    for (int rb = 0; rb < TB; ++rb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) x[rb][v] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < NS0; ++ks)
 #pragma unroll
@@ -264,6 +282,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
+    // wave B: the reads of delta, the start of x, follow the last fragment of the gradient product
+    if constexpr (RB) __builtin_amdgcn_sched_group_barrier(0x100, 4 * TB, 0);
 #pragma unroll
     for (int m = 0; m < NS; ++m) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -305,20 +325,16 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
                                       x[rb][8 * jj + 4], x[rb][8 * jj + 5], x[rb][8 * jj + 6], x[rb][8 * jj + 7]);
     }
   };
-  // B: x = dP of the tile in `stage`, P from the exchange buffer -> dS / scale in frag (bf16), one
-  // 32-row block at a time (the temporaries of a block are dead before the next one is read).
+  // B: x = delta - dP of the tile in `stage`, P from the exchange buffer -> -dS / scale in frag (bf16),
+  // one 32-row block at a time (the temporaries of a block are dead before the next one is read).
   auto make_ds = [&](const char* stage) __attribute__((always_inline)) {
-    const float* delta_s = reinterpret_cast<const float*>(stage + kOffStat) + kBM;
 #pragma unroll
     for (int rb = 0; rb < TB; ++rb) {
-      f32x4 pr[4], d4[4];
+      f32x4 pr[4];
 #pragma unroll
-      for (int b4 = 0; b4 < 4; ++b4) {
-        pr[b4] = *reinterpret_cast<const f32x4*>(exch + ((rb * 4 + b4) * 64 + lane) * 16);
-        d4[b4] = *reinterpret_cast<const f32x4*>(delta_s + 32 * rb + 8 * b4 + 4 * g);
-      }
+      for (int b4 = 0; b4 < 4; ++b4) pr[b4] = *reinterpret_cast<const f32x4*>(exch + ((rb * 4 + b4) * 64 + lane) * 16);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) x[rb][v] = pr[v >> 2][v & 3] * (x[rb][v] - d4[v >> 2][v & 3]);
+      for (int v = 0; v < 16; ++v) x[rb][v] = pr[v >> 2][v & 3] * x[rb][v];
 #pragma unroll
       for (int jj = 0; jj < 2; ++jj)
         frag[2 * rb + jj] = to_bf16x8(x[rb][8 * jj], x[rb][8 * jj + 1], x[rb][8 * jj + 2], x[rb][8 * jj + 3],
@@ -394,7 +410,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
   // ---- epilogue: wave A stores dV, wave B stores dK (times scale), for key row `key`, features
   // 32*o + 8*b4 + 4*g ..+3
   if (key < p.Skv) {
-    const float f = role_b ? p.scale : 1.f;
+    const float f = role_b ? -p.scale : 1.f;  // wave B accumulated -dK / scale
     const int d = role_b ? k_head : kDV;
     const int nblk = role_b ? k_head / 32 : DVB;
     const int64_t row_stride = role_b ? k_row_stride : v_row_stride;

@@ -1,7 +1,7 @@
 // Query-gradient kernel for head dims (128, 128) on gfx950 that reads dS instead of recomputing it:
 // dQ = scale * dS K (pithtrain/operators/mla/triton.py:205-266, the last product of the loop body),
-// with dS = P*(dP - delta) taken, already rounded to bf16, from the images that the dK/dV kernel of
-// attn_bwd_dkdv_d128.hip leaves in p.ds (layout documented there). The two score products that the
+// with dS = P*(dP - delta) taken, already rounded to bf16 and with its sign flipped, from the images
+// that the dK/dV kernel of attn_bwd_dkdv_d128.hip leaves in p.ds (layout documented there). The two score products that the
 // other dQ kernels repeat are gone; the price is one trip of dS through memory, so this kernel is
 // bound by the rate at which it can stream the images, not by the matrix pipe.
 //
@@ -224,6 +224,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
   for (; s < n_steps_wg; ++s) step(s, std::false_type{});
 
   OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * DQK;
+  const float sc = -p.scale;  // the images hold -dS (the writer forms delta - dP)
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb) {
     const int qrow = q_wave0 + 32 * rb + c;
@@ -233,8 +234,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
       for (int o = 0; o < DB; ++o)
 #pragma unroll
         for (int b4 = 0; b4 < 4; ++b4)
-          store4<OutT>(dst + 32 * o + 8 * b4 + 4 * g, acc[rb][o][4 * b4] * p.scale, acc[rb][o][4 * b4 + 1] * p.scale,
-                       acc[rb][o][4 * b4 + 2] * p.scale, acc[rb][o][4 * b4 + 3] * p.scale, p.accumulate != 0);
+          store4<OutT>(dst + 32 * o + 8 * b4 + 4 * g, acc[rb][o][4 * b4] * sc, acc[rb][o][4 * b4 + 1] * sc,
+                       acc[rb][o][4 * b4 + 2] * sc, acc[rb][o][4 * b4 + 3] * sc, p.accumulate != 0);
     }
   }
 }

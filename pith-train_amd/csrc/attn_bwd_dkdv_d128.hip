@@ -9,7 +9,7 @@
 // What differs from the general kernel (all of it measured to matter on the device):
 //   - query tiles are 64 rows, so a wave issues 32 MFMAs between synchronisations;
 //   - Q / dO tiles and the lse / delta rows go global -> LDS directly (global_load_lds) into a
-//     ring of three stages, requested one interval ahead; tiles are packed and swizzled;
+//     ring of three stages, requested one interval ahead by the B waves; tiles are packed and swizzled;
 //   - B runs ONE TILE BEHIND A. In interval i wave A computes dV(i-1), S(i), P(i); wave B
 //     computes dS(i-1), dK(i-1), dP(i);
 //   - A runs [matrix block | vector block], B runs [vector block | matrix block], with a
@@ -89,26 +89,27 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   const int m_first = CAUSAL ? min(kv_wg0 / kBM, m_end) : 0;
   const int n_iter = (m_end - m_first) * heads_per_part;
 
-  // ---- requests
-  DirectTile128<kBM, kThreads> mover;
-  mover.init(q_row_bytes, wave, lane);
+  // ---- requests: issued by the four B waves only (their vector block, dS, is the shorter one: measured
+  // 2 % faster than sharing the requests among all eight waves)
+  DirectTile128<kBM, kThreads / 2> mover;
+  mover.init(q_row_bytes, pair, lane);
   const char* q_base = reinterpret_cast<const char*>(p.q + b * p.q_bs);
   const char* do_base = reinterpret_cast<const char*>(p.dout + b * p.dout_bs);
   TileCursor req = {hq0, m_first};
   auto request = [&](char* stage) __attribute__((always_inline)) {
     const int row0 = req.mt * kBM;
     const int64_t head_off = (int64_t)req.hq * kD * 2 + (int64_t)row0 * q_row_bytes;
-    mover.issue(q_base + head_off, p.Sq - row0, stage, wave, lane);
-    mover.issue(do_base + head_off, p.Sq - row0, stage + kTile, wave, lane);
-    if (wave < 2) {  // wave 0 fetches the 64 lse values of the tile's rows, wave 1 the 64 delta values
+    mover.issue(q_base + head_off, p.Sq - row0, stage, pair, lane);
+    mover.issue(do_base + head_off, p.Sq - row0, stage + kTile, pair, lane);
+    if (pair < 2) {  // pair 0 fetches the 64 lse values of the tile's rows, pair 1 the 64 delta values
       int row = row0 + lane;
       row = row < p.Sq ? row : p.Sq - 1;
-      const float* src = (wave == 0 ? p.lse : p.delta) + b * p.lse_bs + (int64_t)req.hq * p.lse_hs + row;
-      load_lds4(src, stage + 2 * kTile + wave * kBM * 4);
+      const float* src = (pair == 0 ? p.lse : p.delta) + b * p.lse_bs + (int64_t)req.hq * p.lse_hs + row;
+      load_lds4(src, stage + 2 * kTile + pair * kBM * 4);
     }
     req.advance(m_first, m_end);
   };
-  if (n_iter > 0) request(smem);
+  if (n_iter > 0 && role_b) request(smem);
 
   // stationary fragments: K rows for wave A, V rows for wave B
   bf16x8 stat[KS];
@@ -338,7 +339,6 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
     if (!ROLE_B) {
       straight_product(smem + off_cur, role_tag);
       __syncthreads();
-      if (n_iter > 1) request(smem + off_next);
       make_p(smem + off_cur, cur.mt);
     } else {
       if (n_iter > 1) request(smem + off_next);
@@ -353,7 +353,6 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
       if (!ROLE_B) {
         matrix_block(stage_prev, stage_cur, role_tag);
         __syncthreads();  // B has read P(i-1); the matrix pipe passes to B
-        if (will_request) request(smem + off_next);
         make_p(stage_cur, cur.mt);
       } else {
         if (will_request) request(smem + off_next);

@@ -123,32 +123,35 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
   const int m_first = CAUSAL ? min(kv_wg0 / kBM, m_end) : 0;
   const int n_iter = (m_end - m_first) * heads_per_part;
 
-  // ---- requests
-  DirectTile128<kBM, kThreads> q_mover, o_mover;
-  DirectExtra<kBM / 2> e_mover;
-  q_mover.init(q_row_bytes, wave, lane);
-  o_mover.init(do_row_bytes, wave, lane);
-  e_mover.init(q_row_bytes, wave, lane);
+  // ---- requests: issued by the four B waves only (their vector block, dS, is the shorter one)
+  using Extra = DirectExtra<kBM / 2>;
+  DirectTile128<kBM, kThreads / 2> q_mover, o_mover;
+  Extra e_mover[2];  // LDS rows 4*pair .. +3 and, where the extra tile has them, 4*(pair + 4) .. +3
+  q_mover.init(q_row_bytes, pair, lane);
+  o_mover.init(do_row_bytes, pair, lane);
+  e_mover[0].init(q_row_bytes, pair, lane);
+  e_mover[1].init(q_row_bytes, pair + 4, lane);
   const char* q_base = reinterpret_cast<const char*>(p.q + b * p.q_bs);
   const char* do_base = reinterpret_cast<const char*>(p.dout + b * p.dout_bs);
   TileCursor req = {hq0, m_first};
   auto request = [&](char* stage) __attribute__((always_inline)) {
     const int row0 = req.mt * kBM;
     const char* q_src = q_base + (int64_t)req.hq * kDQ * 2 + (int64_t)row0 * q_row_bytes;
-    q_mover.issue(q_src, p.Sq - row0, stage, wave, lane);
-    o_mover.issue(do_base + (int64_t)req.hq * kDV * 2 + (int64_t)row0 * do_row_bytes, p.Sq - row0, stage + kOffO, wave, lane);
-    if (wave < DirectExtra<kBM / 2>::kWaves) e_mover.issue(q_src, p.Sq - row0, stage + kOffExtra, wave, lane);
+    q_mover.issue(q_src, p.Sq - row0, stage, pair, lane);
+    o_mover.issue(do_base + (int64_t)req.hq * kDV * 2 + (int64_t)row0 * do_row_bytes, p.Sq - row0, stage + kOffO, pair, lane);
+    e_mover[0].issue(q_src, p.Sq - row0, stage + kOffExtra, pair, lane);
+    if constexpr (Extra::kWaves > 4) e_mover[1].issue(q_src, p.Sq - row0, stage + kOffExtra, pair + 4, lane);
     // the tile's lse and delta rows: [lse kBM | delta kBM] floats, 64 per wavefront instruction
-    if (TB == 1 ? wave == 4 : wave < 2) {
-      const int idx = TB == 1 ? lane : wave * 64 + lane;  // position in the stats area
+    if (TB == 1 ? pair == 0 : pair < 2) {
+      const int idx = TB == 1 ? lane : pair * 64 + lane;  // position in the stats area
       int row = row0 + (idx & (kBM - 1));
       row = row < p.Sq ? row : p.Sq - 1;
       const float* src = (idx < kBM ? p.lse : p.delta) + b * p.lse_bs + (int64_t)req.hq * p.lse_hs + row;
-      load_lds4(src, stage + kOffStat + (TB == 1 ? 0 : wave * 256));
+      load_lds4(src, stage + kOffStat + (TB == 1 ? 0 : pair * 256));
     }
     req.advance(m_first, m_end);
   };
-  if (n_iter > 0) request(smem);
+  if (n_iter > 0 && role_b) request(smem);
 
   // stationary fragments: K rows for wave A (12), V rows for wave B (8)
   bf16x8 stat[KS];
@@ -366,7 +369,6 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
     if (!ROLE_B) {
       straight_product(smem + off_cur, role_tag);
       __syncthreads();
-      if (n_iter > 1) request(smem + off_next);
       make_p(smem + off_cur, cur.mt);
     } else {
       if (n_iter > 1) request(smem + off_next);
@@ -381,7 +383,6 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
       if (!ROLE_B) {
         matrix_block(stage_prev, stage_cur, role_tag);
         __syncthreads();  // B has read P(i-1); the matrix pipe passes to B
-        if (will_request) request(smem + off_next);
         make_p(stage_cur, cur.mt);
       } else {
         if (will_request) request(smem + off_next);

@@ -54,11 +54,11 @@ FROM_PROFILES = {
     "note": "quoted from committed rocprofv3 summaries, not measured in this run",
     "attn_bwd_dkdv_d128_kernel<non-causal>": {
         "file": "profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt",
-        # with the dS stores: 215.6 MB fetched + 2281.7 MB written (2147.5 MB of dS, 67.1 MB of head-split partials...)
-        "hbm_bytes_per_launch": 2_430_000_000,
-        "hbm_bytes_per_launch_without_ds_stores": 282_700_000,  # 215.6 MB fetched + 67.1 MB written
+        # with the dS stores: 153.4 MB fetched + 2169.9 MB written (2147.5 MB of dS, the rest dK / dV or their head-split partials)
+        "hbm_bytes_per_launch": 2_323_000_000,
+        "hbm_bytes_per_launch_without_ds_stores": 175_700_000,  # 153.4 MB fetched + 22.4 MB written (mean of the three launches)
         "mfma_file": "profiles/attn_kernels_mfma_lds_counters.txt",
-        "mfma_busy_fraction": 0.54,  # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs); 0.615 without the stores
+        "mfma_busy_fraction": 0.58,  # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs); 0.68 without the stores
         "sustained_clock_ghz": 1.75,  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration (2.4 GHz nominal); 1.85 without the stores
     },
     "combine_front_kernel": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_per_launch": COMBINE_TRAFFIC},

@@ -322,10 +322,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
     constexpr bool ROLE_B = decltype(role_tag)::value;
     TileCursor cur = {hq0, m_first}, done = cur;  // tiles i and i-1 of interval i
     int off_prev = 2 * kStage, off_cur = 0, off_next = kStage;
-    auto end_interval = [&]() __attribute__((always_inline)) {
+    auto end_interval = [&](bool stored) __attribute__((always_inline)) {
       // the tile requested in this interval has landed. Vector memory operations complete in issue
-      // order, and wave B issued its four dS stores after the request: they may stay in flight.
-      if (ROLE_B && EMIT_DS) __builtin_amdgcn_s_waitcnt(0x0F74);
+      // order, and where wave B issued its four dS stores after the request (every interval but the
+      // first) they may stay in flight.
+      if (ROLE_B && EMIT_DS && stored) __builtin_amdgcn_s_waitcnt(0x0F74);
       else __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
       done = cur;
@@ -345,7 +346,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
       __syncthreads();
       straight_product(smem + off_cur, role_tag);
     }
-    end_interval();
+    end_interval(false);
     for (int i = 1; i < n_iter; ++i) {
       const char* stage_cur = smem + off_cur;
       const char* stage_prev = smem + off_prev;
@@ -360,7 +361,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
         __syncthreads();
         matrix_block(stage_prev, stage_cur, role_tag);
       }
-      end_interval();
+      end_interval(true);
     }
     // interval n_iter
     if (!ROLE_B) {

@@ -174,12 +174,29 @@ def bench_recompute(torch, dev_inputs, steps, warmup):
     }  # fmt: skip
 
 
+def handover_scratch_bytes(cfg, dev):
+    """Bytes of dS hand-over scratch the ring backward takes per non-causal ring step of `cfg` (0: it recomputes)."""
+    from pithtrain_amd.operators.mla import hip
+    from pithtrain_amd.operators.ring_attention.local import ring_schedule
+
+    q, ks, vs, _ = dev
+    most = 0
+    for s in ring_schedule(cfg.rank, cfg.cp, cfg.s_local, LAYOUT):
+        if not s.causal:
+            rows = slice(s.kv_rows[0], s.kv_rows[1])
+            need = hip.attn_bwd_ds_bytes(q[:, s.q_rows[0] : s.q_rows[1]], ks[s.kv_rank][:, rows], vs[s.kv_rank][:, rows])
+            most = max(most, need if 0 < need <= hip.DS_BUFFER_LIMIT_BYTES else 0)
+    return most
+
+
 def bench_other_config(torch, device, cfg, steps, warmup):
     _, dev = cfg.make_inputs(torch, device)
     ms_step, ms_fwd, ms_bwd, _, _ = time_ring_share(torch, cfg, dev, steps, warmup)
+    out = ring_summary(cfg, ms_step, ms_fwd, ms_bwd)
+    out["ds_handover_scratch_bytes_per_ring_step"] = handover_scratch_bytes(cfg, dev)
     del dev
     torch.cuda.empty_cache()
-    return ring_summary(cfg, ms_step, ms_fwd, ms_bwd)
+    return out
 
 
 def bench_ring(torch, args, dev_inputs):

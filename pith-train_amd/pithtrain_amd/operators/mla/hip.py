@@ -159,7 +159,7 @@ def _set_ds(args, ds: torch.Tensor, like: torch.Tensor) -> None:
 # Above this size the hand-over buffer is not worth its memory: the two backward calls recompute.
 # The hand-over makes the backward 3-6 % faster at the price of Sq*Skv*Hq*B*2 bytes of scratch while the two
 # kernels run (2 GiB per ring step at 32 heads and 8192 x 4096 rows, 16 GiB at 64 heads and 16384 x 8192).
-DS_BUFFER_LIMIT_BYTES = int(float(os.environ.get("PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB", "4")) * (1 << 30))
+DS_BUFFER_LIMIT_BYTES = int(float(os.environ.get("PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB", "16")) * (1 << 30))
 _DS_ROWS_PER_WORKGROUP = 512  # query rows a workgroup of the dS-reading dQ kernel owns
 _compute_units = {}
 

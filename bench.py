@@ -175,17 +175,16 @@ def bench_recompute(torch, dev_inputs, steps, warmup):
 
 
 def handover_scratch_bytes(cfg, dev):
-    """Bytes of dS hand-over scratch the ring backward takes per non-causal ring step of `cfg` (0: it recomputes)."""
+    """Largest dS hand-over scratch the ring backward takes in a ring step of `cfg` (0: it recomputes in all of them)."""
     from pithtrain_amd.operators.mla import hip
     from pithtrain_amd.operators.ring_attention.local import ring_schedule
 
     q, ks, vs, _ = dev
     most = 0
     for s in ring_schedule(cfg.rank, cfg.cp, cfg.s_local, LAYOUT):
-        if not s.causal:
-            rows = slice(s.kv_rows[0], s.kv_rows[1])
-            need = hip.attn_bwd_ds_bytes(q[:, s.q_rows[0] : s.q_rows[1]], ks[s.kv_rank][:, rows], vs[s.kv_rank][:, rows])
-            most = max(most, need if 0 < need <= hip.DS_BUFFER_LIMIT_BYTES else 0)
+        rows = slice(s.kv_rows[0], s.kv_rows[1])
+        need = hip.attn_bwd_ds_bytes(q[:, s.q_rows[0] : s.q_rows[1]], ks[s.kv_rank][:, rows], vs[s.kv_rank][:, rows], s.causal)
+        most = max(most, need if 0 < need <= hip.DS_BUFFER_LIMIT_BYTES else 0)
     return most
 
 
@@ -469,6 +468,7 @@ def main():
     recompute = None
     if not args.no_extra_configs and handover_on:
         recompute = bench_recompute(torch, dev_inputs, args.steps, args.warmup)
+    scratch = handover_scratch_bytes(QWEN3, dev_inputs) if handover_on else 0
     del dev_inputs
     torch.cuda.empty_cache()
     fwd_flops, bwd_flops = flops_per_step()
@@ -544,7 +544,7 @@ def main():
         "ds_handover": {
             "on": handover_on,
             "what": "the dK/dV kernel hands its dS tiles to the dQ kernel (5 matrix products executed instead of 7)",
-            "scratch_bytes_per_ring_step": HQ * S_LOCAL * (S_LOCAL // 2) * 2 if handover_on else 0,
+            "scratch_bytes_per_ring_step": scratch,
             "recompute_backward": recompute,
         },
         "mla16k": mla16k,

@@ -209,7 +209,8 @@ int64_t pith_attn_bwd_dkdv_workspace_bytes(const pith_attn_bwd_args* args);
  * and a pith_attn_bwd_dq call with the SAME shapes, strides, causal flag and `ds`, enqueued after
  * it on the same stream, computes dQ = scale * dS K from those tiles without recomputing the
  * scores: the backward then executes 5 matrix products instead of 7, at the price of
- * Sq*Skv*Hq*B*2 bytes written and read once. Results agree with the recomputing dQ kernel up to
+ * Sq*Skv*Hq*B*2 bytes written and read once (a causal call keeps only the tiles at or below the
+ * diagonal: about half). Results agree with the recomputing dQ kernel up to
  * fp32 summation order (the dS values are the same bf16 numbers). The buffer holds nothing of
  * value after the dQ call. Returns the bytes needed, or 0 when the shape has no hand-over path
  * (head dims other than (128,128)); with ds == NULL or a buffer that is too small both calls

@@ -30,10 +30,23 @@ struct BwdParams {
   int64_t k_pe_bs, k_pe_rs;
   float* ws_dkpe;
   // dS hand-over from the dK/dV kernel to the dQ kernel (head dims 128/128): bf16 images, 16 KB per
-  // (batch, query head, 64-row query tile, 128-key block); ds_qt / ds_kb = number of such tiles / blocks
+  // (batch, query head, 64-row query tile, 128-key block); ds_qt / ds_kb = number of such tiles / blocks.
+  // Without a causal mask a head holds ds_qt x ds_kb of them, query tile by query tile; under the mask
+  // only the blocks a tile can see are kept (tile t: its first t/2 + 1 key blocks, see ds_tile_start).
+  // ds_hs = bytes per (batch, head).
   char* ds;
   int ds_qt, ds_kb;
+  int64_t ds_hs;
 };
+
+constexpr int kDsBlockBytes = 4 * 4096;  // one (query tile, key block): four wave-pair images
+// Number of 16 KB blocks that precede query tile t within a head.
+template <bool CAUSAL>
+__host__ __device__ __forceinline__ int64_t ds_tile_start(int t, int ds_kb) {
+  if (!CAUSAL) return (int64_t)t * ds_kb;
+  const int64_t a = t >> 1;  // tiles 2a and 2a + 1 see a + 1 key blocks each
+  return (t & 1) ? (a + 1) * (a + 1) : a * (a + 1);
+}
 
 // Stores 4 consecutive output features held by one lane; OutT is __bf16 or float.
 template <typename OutT>

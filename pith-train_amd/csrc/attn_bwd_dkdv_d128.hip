@@ -51,7 +51,7 @@ struct TileCursor {
 // EMIT_DS: wave B also stores every dS tile it forms (bf16, as -dS before the factor `scale`) to p.ds for
 // the dQ kernel of attn_bwd_dq_ds.hip, which then needs no score recomputation. Layout of p.ds:
 // one 4 KB image per (batch, query head, 64-row query tile, 128-key block, wave pair), in that
-// order; an image is the four bf16x8 fragments of the pair's B wave as they sit in registers,
+// order (under the causal mask only the key blocks a query tile can see: ds_tile_start); an image is the four bf16x8 fragments of the pair's B wave as they sit in registers,
 // 1 KB per 16-row step j, the 16 bytes of lane (g, c) at g*512 + ((c ^ 8g ^ 4(j&1)) << 4) (the
 // XOR terms make the reader's transposing LDS reads conflict-free). Keys at or beyond Skv hold 0
 // (their P is masked to 0).
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
                                       x[rb][8 * jj + 4], x[rb][8 * jj + 5], x[rb][8 * jj + 6], x[rb][8 * jj + 7]);
     }
     if constexpr (EMIT_DS) {
-      char* img = ds_wg + (((int64_t)(b * p.Hq + tile.hq) * p.ds_qt + tile.mt) * p.ds_kb) * (4 * 4096);
+      char* img = ds_wg + (int64_t)(b * p.Hq + tile.hq) * p.ds_hs + ds_tile_start<CAUSAL>(tile.mt, p.ds_kb) * kDsBlockBytes;
       int off = (g << 9) + ((c ^ (g << 3)) << 4);  // recomputed per tile: no register is held across the interval
       asm volatile("" : "+v"(off));
 #pragma unroll

@@ -293,12 +293,16 @@ BwdParams make_bwd_params(const pith_attn_bwd_args* a) {
   p.ds = nullptr;
   p.ds_qt = (int)((a->Sq + 63) / 64);
   p.ds_kb = (int)((a->Skv + kDkdvBlockN - 1) / kDkdvBlockN);
+  p.ds_hs = (a->causal ? ds_tile_start<true>(p.ds_qt, p.ds_kb) : ds_tile_start<false>(p.ds_qt, p.ds_kb)) * kDsBlockBytes;
   return p;
 }
 
 int64_t ds_bytes_for(const pith_attn_bwd_args* a) {
   if (!a || a->Dqk != 128 || a->Dv != 128 || a->k_pe || a->B <= 0 || a->Hq <= 0 || a->Sq <= 0 || a->Skv <= 0) return 0;
-  return a->B * a->Hq * ((a->Sq + 63) / 64) * ((a->Skv + kDkdvBlockN - 1) / kDkdvBlockN) * (int64_t)(4 * 4096);
+  const int qt = (int)((a->Sq + 63) / 64), kb = (int)((a->Skv + kDkdvBlockN - 1) / kDkdvBlockN);
+  // a causal call (Sq == Skv) keeps only the key blocks at or below the diagonal of every query tile
+  const int64_t blocks = a->causal ? ds_tile_start<true>(qt, kb) : ds_tile_start<false>(qt, kb);
+  return a->B * a->Hq * blocks * kDsBlockBytes;
 }
 
 }  // namespace pith

@@ -95,7 +95,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
   // consecutive in s; the rows' part starts 1 KB per 16 rows into each image
   auto images_of = [&](int q0) __attribute__((always_inline)) {
     const int mt = min(q0 >> 6, p.ds_qt - 1);
-    return p.ds + (((int64_t)(b * p.Hq + h) * p.ds_qt + mt) * p.ds_kb) * (4 * 4096) + (q0 & 63) * 64;
+    return p.ds + (int64_t)(b * p.Hq + h) * p.ds_hs + ds_tile_start<CAUSAL>(mt, p.ds_kb) * kDsBlockBytes + (q0 & 63) * 64;
   };
 
   // ---- requests. Waves 0..3: K tiles. Waves 4..7: the dS parts of waves w-4 and w.

@@ -140,11 +140,12 @@ def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe=None) -> _C
     )  # fmt: skip
 
 
-def attn_bwd_ds_bytes(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> int:
+def attn_bwd_ds_bytes(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool = False) -> int:
     """Bytes of the dS hand-over buffer for one chunk pair (0: these head dims have no hand-over path,
-    both backward calls then recompute the scores)."""
+    both backward calls then recompute the scores). A causal pair needs about half: only the tiles at
+    or below the diagonal are kept."""
     b, sq, hq, d_q = q.shape
-    args = _C.AttnBwdArgs(B=b, Sq=sq, Skv=k.shape[1], Hq=hq, Hkv=k.shape[2], Dqk=d_q, Dv=v.shape[-1])
+    args = _C.AttnBwdArgs(B=b, Sq=sq, Skv=k.shape[1], Hq=hq, Hkv=k.shape[2], Dqk=d_q, Dv=v.shape[-1], causal=int(bool(causal)))
     return int(_C.lib().pith_attn_bwd_ds_bytes(_C.byref(args)))
 
 
@@ -158,8 +159,9 @@ def _set_ds(args, ds: torch.Tensor, like: torch.Tensor) -> None:
 
 # Above this size the hand-over buffer is not worth its memory: the two backward calls recompute.
 # The hand-over makes the backward 3-6 % faster at the price of Sq*Skv*Hq*B*2 bytes of scratch while the two
-# kernels run (2 GiB per ring step at 32 heads and 8192 x 4096 rows, 16 GiB at 64 heads and 16384 x 8192).
-DS_BUFFER_LIMIT_BYTES = int(float(os.environ.get("PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB", "16")) * (1 << 30))
+# kernels run (2 GiB per ring step at 32 heads and 8192 x 4096 rows, 16 GiB at 64 heads and 16384 x 8192; a
+# causal pair needs half of the full rectangle plus its diagonal blocks: 16.1 GiB at 64 heads and 16384 rows).
+DS_BUFFER_LIMIT_BYTES = int(float(os.environ.get("PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB", "17")) * (1 << 30))
 _DS_ROWS_PER_WORKGROUP = 512  # query rows a workgroup of the dS-reading dQ kernel owns
 _compute_units = {}
 
@@ -173,12 +175,12 @@ def _device_compute_units(device: torch.device) -> int:
     return _compute_units[idx]
 
 
-def ds_buffer(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+def ds_buffer(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool = False):
     """A dS hand-over buffer for one chunk pair from torch's caching allocator, or None when the
     shape has no hand-over path, the buffer would exceed DS_BUFFER_LIMIT_BYTES, or the dS-reading dQ
     kernel would have fewer workgroups than the device has compute units (the recomputing kernels
     use smaller workgroups and then win)."""
-    need = attn_bwd_ds_bytes(q, k, v)
+    need = attn_bwd_ds_bytes(q, k, v, causal)
     if need == 0 or need > DS_BUFFER_LIMIT_BYTES:
         return None
     b, sq, hq, _ = q.shape
@@ -194,7 +196,7 @@ def attn_bwd_dkdv_into(
     """dk, dv <- (or +=, with accumulate) the gradients of this chunk pair; bf16 or fp32 outputs.
     With k_pe (see attn_fwd_into) dk is the gradient of k_nope and dk_pe [b, skv, 64] (contiguous rows,
     same dtype as dk) receives the gradient of k_pe, summed over heads in head order.
-    ds: uint8 buffer of attn_bwd_ds_bytes(q, k, v) bytes; the kernel leaves its dS tiles there for an
+    ds: uint8 buffer of attn_bwd_ds_bytes(q, k, v, causal) bytes; the kernel leaves its dS tiles there for an
     attn_bwd_dq_into call on the same chunk pair with the same buffer."""
     args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe)
     _set_ds(args, ds, q)
@@ -313,7 +315,7 @@ def _attn_bwd_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Ten
     q, k, v, o, dout = q.contiguous(), k.contiguous(), v.contiguous(), o.contiguous(), dout.contiguous()
     delta = _mla_bwd_preprocess(o, dout)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    ds = ds_buffer(q, k, v)
+    ds = ds_buffer(q, k, v, causal)
     attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, softmax_scale, causal, ds=ds)
     attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, softmax_scale, causal, ds=ds)
     return dq, dk, dv

@@ -255,7 +255,7 @@ class RingBackward:
         pes = _pe_rows(k_pe_j, st.kv_rows)
         # The dK/dV kernel leaves its dS tiles in `hand` for the dQ kernel, which then skips the score
         # recomputation (head dims 128/128; None otherwise: both kernels recompute).
-        hand = ds_buffer(qs, ks, vs) if pes is None else None
+        hand = ds_buffer(qs, ks, vs, st.causal) if pes is None else None
         attn_bwd_dkdv_into(qs, ks, vs, ds, ls, dl, _rows(dk_j, st.kv_rows), _rows(dv_j, st.kv_rows),
                            self.scale, st.causal, accumulate=add_to is not None, k_pe=pes,
                            dk_pe=_pe_rows(dk_pe_j, st.kv_rows), ds=hand)  # fmt: skip

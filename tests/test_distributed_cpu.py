@@ -42,7 +42,7 @@ def _install_cpu_stand_ins():
         rdq, _, _ = R.chunk_bwd(q, full_key(k, k_pe), v, dout, lse.double(), delta.double(), scale, causal)
         dq.copy_(dq.double() + rdq if accumulate else rdq)
 
-    def ds_buffer(q, k, v):  # no dS hand-over between the stand-ins
+    def ds_buffer(q, k, v, causal=False):  # no dS hand-over between the stand-ins
         return None
 
     def combine_into(out1, lse1, out2, lse2, out, lse_out, base=0):

@@ -56,8 +56,11 @@ def _run(gpu, causal, shape, dq_dtype, dqk=128):
     attn_bwd_dkdv_into(qd, kd, vd, dod, lse, delta, dk0, dv0, scale, causal)
     attn_bwd_dq_into(qd, kd, vd, dod, lse, delta, dq0, scale, causal)
 
-    need = attn_bwd_ds_bytes(qd, kd, vd)
-    assert need == shape[0] * shape[3] * ((shape[1] + 63) // 64) * ((shape[2] + 127) // 128) * 16384
+    need = attn_bwd_ds_bytes(qd, kd, vd, causal)
+    n_qt, n_kb = (shape[1] + 63) // 64, (shape[2] + 127) // 128
+    # 16 KB per (64-row query tile, 128-key block); under the mask tile t keeps its first t // 2 + 1 key blocks
+    blocks = sum(t // 2 + 1 for t in range(n_qt)) if causal else n_qt * n_kb
+    assert need == shape[0] * shape[3] * blocks * 16384
     # poisoned buffer: whatever the dQ kernel reads must have been written by the dK/dV kernel
     ds = torch.full((need,), 0x7F, dtype=torch.uint8, device=gpu)
     dk1, dv1 = torch.empty_like(kd), torch.empty_like(vd)
@@ -97,7 +100,7 @@ def test_small_buffer_falls_back_to_recomputation(gpu):
     delta = _mla_bwd_preprocess(o, dod)
     dq0, dq1 = torch.empty_like(qd), torch.empty_like(qd)
     attn_bwd_dq_into(qd, kd, vd, dod, lse, delta, dq0, scale, True)
-    small = torch.zeros(attn_bwd_ds_bytes(qd, kd, vd) - 1024, dtype=torch.uint8, device=gpu)
+    small = torch.zeros(attn_bwd_ds_bytes(qd, kd, vd, True) - 1024, dtype=torch.uint8, device=gpu)
     attn_bwd_dq_into(qd, kd, vd, dod, lse, delta, dq1, scale, True, ds=small)
     assert torch.equal(dq0, dq1)
     # head dims without a hand-over path report 0 bytes and get no buffer
@@ -128,9 +131,9 @@ def test_ring_share_uses_the_handover(gpu, layout, monkeypatch):
 
     calls = []
 
-    def always(q, k, v):  # the default policy would decline a share this small
+    def always(q, k, v, causal=False):  # the default policy would decline a share this small
         calls.append(1)
-        return torch.empty(attn_bwd_ds_bytes(q, k, v), dtype=torch.uint8, device=q.device)
+        return torch.empty(attn_bwd_ds_bytes(q, k, v, causal), dtype=torch.uint8, device=q.device)
 
     monkeypatch.setattr(L, "ds_buffer", always)
     dq1, dk1, dv1 = run()

@@ -29,6 +29,9 @@ SHAPES = [
     (1, 333, 333, 4, 2),      # ragged last query tile and key block
     (1, 1000, 1000, 2, 1),
     (1, 2048, 2048, 16, 2),   # head split of the dK/dV kernel
+    (1, 65, 65, 2, 2),        # one row beyond a query tile: two tiles, one key block
+    (1, 129, 129, 4, 1),      # one row beyond a key block
+    (2, 777, 777, 8, 2),
 ]
 NONCAUSAL_SHAPES = SHAPES + [(1, 512, 256, 8, 2), (1, 256, 768, 4, 4), (1, 200, 450, 4, 2), (1, 65, 129, 2, 2)]
 

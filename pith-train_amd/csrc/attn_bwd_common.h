@@ -74,6 +74,40 @@ __device__ __forceinline__ void store4<__bf16>(__bf16* dst, float a0, float a1, 
   *reinterpret_cast<u32x2*>(dst) = w;
 }
 
+// Stores a 32-row block of a result whose accumulators hold it UNtransposed: acc[o][v] is element
+// (row acc_row(v, g), feature 32*o + c) for lane (c, g). For one v the 64 lanes cover two rows x 32 consecutive
+// features: every instruction reads or writes whole 128-byte lines (fp32), where the transposed form (a lane owning
+// one row and 4 consecutive features per access) touches 32 lines with 32 bytes each. `block` = row 0, feature 0 of
+// the block; rows at or beyond `rows_valid` are skipped. With `accumulate` the old values are all read before the
+// first store (row pointers may alias as far as the compiler can tell; it would chain load - store - load otherwise).
+template <typename OutT, int NB>
+__device__ __forceinline__ void store_rows32(OutT* block, int64_t row_stride, int rows_valid, const f32x16 (&acc)[NB],
+                                             float factor, bool accumulate, int c, int g) {
+#pragma clang fp contract(off)  // product rounded, then added: what accumulating into a separate tensor gives
+  float old[16][NB];
+  if (accumulate) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int r = acc_row(v, g);
+      const OutT* src = block + (r < rows_valid ? r : 0) * row_stride + c;
+#pragma unroll
+      for (int o = 0; o < NB; ++o) old[v][o] = (float)src[32 * o];
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int r = acc_row(v, g);
+    if (r < rows_valid) {
+      OutT* dst = block + r * row_stride + c;
+#pragma unroll
+      for (int o = 0; o < NB; ++o) {
+        float x = acc[o][v] * factor;
+        if (accumulate) x += old[v][o];
+        dst[32 * o] = (OutT)x;
+      }
+    }
+  }
+}
 
 // dK/dV kernels: a workgroup owns kDkdvBlockN key rows (the grid and the head split depend on it).
 constexpr int kDkdvBlockN = 128;

@@ -17,9 +17,11 @@
 // also waiting for every image it requested before that tile; therefore waves 0..3 request the K
 // tiles and nothing else, and waves 4..7 request the images of all eight waves (each its own and that
 // of wave w - 4). Every wave waits for its own requests and the step's barrier publishes them.
-// dQ^T += K^T dS^T: K^T fragments come from transposing reads of the K tile and serve both 32-row
-// blocks of the wave's tile, dS^T fragments from transposing reads of the image, in the same key slot
-// order.
+// dQ += dS K: K fragments (B operands: 32 features x 16 keys) come from transposing reads of the K tile
+// and serve both 32-row blocks of the wave's tile, dS fragments (A operands: 32 query rows x 16 keys)
+// from transposing reads of the image, in the same key slot order. The accumulators therefore hold
+// dQ untransposed (a lane owns one feature column of 16 rows) and the epilogue reads and writes whole
+// 128-byte lines (store_rows32).
 // With 192-feature keys the same scheme was measured not to pay: a workgroup then holds accumulators
 // for 256 rows only, K is 43 % of the bytes a compute unit requests, and the kernel is no faster than
 // recomputing the scores.
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
         const char* kt = stage + ks * 16 * kRowBytes128;
         const bf16x8 a = lds_read_transposed_at(kt + (t_base[0] ^ (o << 6)), kt + (t_base[1] ^ (o << 6)));
 #pragma unroll
-        for (int rb = 0; rb < RBW; ++rb) acc[rb][o] = mfma32(a, dsf[rb], acc[rb][o]);
+        for (int rb = 0; rb < RBW; ++rb) acc[rb][o] = mfma32(dsf[rb], a, acc[rb][o]);
       }
     }
   };
@@ -225,18 +227,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
 
   OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * DQK;
   const float sc = -p.scale;  // the images hold -dS (the writer forms delta - dP)
+  const int64_t row_stride = (int64_t)p.Hq * DQK;
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb) {
-    const int qrow = q_wave0 + 32 * rb + c;
-    if (qrow < p.Sq) {
-      OutT* dst = dqh + qrow * ((int64_t)p.Hq * DQK);
-#pragma unroll
-      for (int o = 0; o < DB; ++o)
-#pragma unroll
-        for (int b4 = 0; b4 < 4; ++b4)
-          store4<OutT>(dst + 32 * o + 8 * b4 + 4 * g, acc[rb][o][4 * b4] * sc, acc[rb][o][4 * b4 + 1] * sc,
-                       acc[rb][o][4 * b4 + 2] * sc, acc[rb][o][4 * b4 + 3] * sc, p.accumulate != 0);
-    }
+    const int row0 = q_wave0 + 32 * rb;
+    store_rows32<OutT, DB>(dqh + row0 * row_stride, row_stride, p.Sq - row0, acc[rb], sc, p.accumulate != 0, c, g);
   }
 }
 

@@ -78,32 +78,37 @@ __device__ __forceinline__ void store4<__bf16>(__bf16* dst, float a0, float a1, 
 // (row acc_row(v, g), feature 32*o + c) for lane (c, g). For one v the 64 lanes cover two rows x 32 consecutive
 // features: every instruction reads or writes whole 128-byte lines (fp32), where the transposed form (a lane owning
 // one row and 4 consecutive features per access) touches 32 lines with 32 bytes each. `block` = row 0, feature 0 of
-// the block; rows at or beyond `rows_valid` are skipped. With `accumulate` the old values are all read before the
-// first store (row pointers may alias as far as the compiler can tell; it would chain load - store - load otherwise).
+// the block; rows at or beyond `rows_valid` are skipped. With `accumulate` the old values of a batch of rows are all read before
+// the batch's first store (row pointers may alias as far as the compiler can tell; it would chain load - store - load
+// otherwise).
 template <typename OutT, int NB>
 __device__ __forceinline__ void store_rows32(OutT* block, int64_t row_stride, int rows_valid, const f32x16 (&acc)[NB],
                                              float factor, bool accumulate, int c, int g) {
 #pragma clang fp contract(off)  // product rounded, then added: what accumulating into a separate tensor gives
-  float old[16][NB];
-  if (accumulate) {
+  constexpr int kBatch = NB > 4 ? 4 : 8;  // accumulator elements per lane and batch: NB * kBatch old values in registers
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int r = acc_row(v, g);
-      const OutT* src = block + (r < rows_valid ? r : 0) * row_stride + c;
+  for (int v0 = 0; v0 < 16; v0 += kBatch) {
+    float old[kBatch][NB];
+    if (accumulate) {
 #pragma unroll
-      for (int o = 0; o < NB; ++o) old[v][o] = (float)src[32 * o];
+      for (int dv = 0; dv < kBatch; ++dv) {
+        const int r = acc_row(v0 + dv, g);
+        const OutT* src = block + (r < rows_valid ? r : 0) * row_stride + c;
+#pragma unroll
+        for (int o = 0; o < NB; ++o) old[dv][o] = (float)src[32 * o];
+      }
     }
-  }
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int r = acc_row(v, g);
-    if (r < rows_valid) {
-      OutT* dst = block + r * row_stride + c;
+    for (int dv = 0; dv < kBatch; ++dv) {
+      const int r = acc_row(v0 + dv, g);
+      if (r < rows_valid) {
+        OutT* dst = block + r * row_stride + c;
 #pragma unroll
-      for (int o = 0; o < NB; ++o) {
-        float x = acc[o][v] * factor;
-        if (accumulate) x += old[v][o];
-        dst[32 * o] = (OutT)x;
+        for (int o = 0; o < NB; ++o) {
+          float x = acc[o][v0 + dv] * factor;
+          if (accumulate) x += old[dv][o];
+          dst[32 * o] = (OutT)x;
+        }
       }
     }
   }

@@ -53,7 +53,9 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   constexpr int kBM = HALF ? 128 : 256;      // query rows per workgroup
   constexpr int kKTile = kTile + (DQK == 192 ? kExtraTile : 0);
   static_assert(DQK == 128 || DQK == 192, "head dims");
-  __shared__ __attribute__((aligned(1024))) char smem[kSlots * (kKTile + kTile)];
+  // the tile rings; the epilogue reuses them to turn the output tile (one area per storing wave)
+  constexpr int kRings = kSlots * (kKTile + kTile), kTurn = (HALF ? kWaves / 2 : kWaves) * kRowsViaLdsBytes<DVB>;
+  __shared__ __attribute__((aligned(1024))) char smem[kRings > kTurn ? kRings : kTurn];
   char* const kbuf = smem;
   char* const vbuf = smem + kSlots * kKTile;
 
@@ -380,7 +382,14 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   float* lse = p.lse + b * p.lse_bs + (int64_t)h * p.lse_hs;
   const float l = pair_sum(l_run);
   const float inv = l > 0.f ? 1.f / l : 0.f;
-  if (qrow < p.Sq) {
+  // O^T sits in the accumulators (a lane owns one query row): turned through LDS so that the stores
+  // cover whole rows. Every wave is past the barrier behind the last tile read (HALF: past the merge).
+  // (Not in the 256-row causal kernel for 192-feature keys, which has no register to spare: the extra
+  // live values of the turned epilogue push spills into its main loop.)
+  if constexpr (!(DQK == 192 && !HALF && CAUSAL)) {
+    char* const turn = smem + (HALF ? (wave & 3) : wave) * kRowsViaLdsBytes<DVB>;
+    store_rows32_via_lds<__bf16, DVB>(turn, oh + q_wave0 * o_row_stride, o_row_stride, p.Sq - q_wave0, oacc, inv, false, lane);
+  } else if (qrow < p.Sq) {
     __bf16* dst = oh + qrow * o_row_stride;
 #pragma unroll
     for (int i = 0; i < DVB; ++i)
@@ -391,8 +400,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
         w[1] = pack_bf16x2(oacc[i][4 * b4 + 2] * inv, oacc[i][4 * b4 + 3] * inv);
         *reinterpret_cast<u32x2*>(dst + 32 * i + 8 * b4 + 4 * g) = w;
       }
-    if (g == 0) lse[qrow] = (l > 0.f) ? __builtin_amdgcn_logf(l) + m_run * p.kappa : -INFINITY;
   }
+  if (qrow < p.Sq && g == 0) lse[qrow] = (l > 0.f) ? __builtin_amdgcn_logf(l) + m_run * p.kappa : -INFINITY;
 }
 
 template <int DQK, bool HALF>

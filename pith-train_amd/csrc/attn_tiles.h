@@ -288,4 +288,74 @@ __device__ __forceinline__ bf16x8 lds_read_transposed_at(const char* lo_addr, co
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Epilogue of the kernels whose accumulators hold their result TRANSPOSED (a lane owns one result
+// row, its registers 4-feature pieces of it: accT[o][v] = R[row c][feature 32*o + acc_row(v, g)] for lane
+// (c, g)). Written straight from that layout a store instruction touches 32 rows with 16 or 32 bytes
+// each, i.e. 32 memory lines, and a compute unit's vector cache keeps only about 64 requests in flight;
+// turned through LDS first, every instruction reads or writes whole rows (2 rows x 512 bytes of fp32 per
+// instruction at 128 features). `lds` is a wave-private area of kRowsViaLdsBytes<NB> bytes (the tile
+// rings are free by then: the caller has passed the barrier behind their last reader); `factor` is this
+// lane's (= this row's) scale; rows at or beyond rows_valid are not written. With `accumulate` all old
+// values are read before the first store.
+template <int NB>
+constexpr int kRowsViaLdsBytes = 32 * (NB * 128 + 16);
+
+template <typename OutT, int NB>
+__device__ __forceinline__ void store_rows32_via_lds(char* lds, OutT* block, int64_t row_stride, int rows_valid,
+                                                     const f32x16 (&accT)[NB], float factor, bool accumulate, int lane) {
+#pragma clang fp contract(off)  // product rounded, then added: what accumulating into a separate tensor gives
+  constexpr int kPitch = NB * 128 + 16;  // bytes; the 16 spread the 32 rows of a column over the banks
+  constexpr int kPieces = NB * 8;        // 16-byte pieces (4 features) per row
+  constexpr int kIters = 32 * kPieces / 64;
+  const int c = lane & 31, g = lane >> 5;
+#pragma unroll
+  for (int o = 0; o < NB; ++o)
+#pragma unroll
+    for (int b4 = 0; b4 < 4; ++b4) {
+      const f32x4 x = {accT[o][4 * b4] * factor, accT[o][4 * b4 + 1] * factor, accT[o][4 * b4 + 2] * factor,
+                       accT[o][4 * b4 + 3] * factor};
+      *reinterpret_cast<f32x4*>(lds + c * kPitch + (32 * o + 8 * b4 + 4 * g) * 4) = x;
+    }
+  // the reads below see the writes above: one wave's LDS operations execute in order
+  f32x4 val[kIters];
+  int row[kIters], piece[kIters];
+#pragma unroll
+  for (int it = 0; it < kIters; ++it) {
+    const int idx = it * 64 + lane;
+    row[it] = idx / kPieces;
+    piece[it] = idx - row[it] * kPieces;
+    val[it] = *reinterpret_cast<const f32x4*>(lds + row[it] * kPitch + piece[it] * 16);
+  }
+  if (accumulate) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      const OutT* src = block + (row[it] < rows_valid ? row[it] : 0) * row_stride + 4 * piece[it];
+      if constexpr (sizeof(OutT) == 4) {
+        val[it] += *reinterpret_cast<const f32x4*>(src);
+      } else {
+        const u32x2 old = *reinterpret_cast<const u32x2*>(src);
+        val[it][0] += bf16lo_to_f32(old[0]);
+        val[it][1] += bf16hi_to_f32(old[0]);
+        val[it][2] += bf16lo_to_f32(old[1]);
+        val[it][3] += bf16hi_to_f32(old[1]);
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < kIters; ++it) {
+    if (row[it] < rows_valid) {
+      OutT* dst = block + row[it] * row_stride + 4 * piece[it];
+      if constexpr (sizeof(OutT) == 4) {
+        *reinterpret_cast<f32x4*>(dst) = val[it];
+      } else {
+        u32x2 w;
+        w[0] = pack_bf16x2(val[it][0], val[it][1]);
+        w[1] = pack_bf16x2(val[it][2], val[it][3]);
+        *reinterpret_cast<u32x2*>(dst) = w;
+      }
+    }
+  }
+}
+
 }  // namespace pith

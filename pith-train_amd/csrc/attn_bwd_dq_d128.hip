@@ -32,7 +32,9 @@ constexpr int kTile = kBN * kRowBytes128;
 template <bool CAUSAL, typename OutT>
 __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p) {
   constexpr int KS = kD / 16, DB = kD / 32;
-  __shared__ __attribute__((aligned(1024))) char smem[(kKSlots + kVSlots) * kTile];
+  // the tile rings; the epilogue reuses the memory to turn the result tile (one area per wave)
+  constexpr int kRings = (kKSlots + kVSlots) * kTile, kTurn = kThreads / 64 * kRowsViaLdsBytes<DB>;
+  __shared__ __attribute__((aligned(1024))) char smem[kRings > kTurn ? kRings : kTurn];
   char* const kbuf = smem;
   char* const vbuf = smem + kKSlots * kTile;
 
@@ -274,16 +276,13 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
     end_interval();
   }
 
+  // dQ^T sits in the accumulators (a lane owns one query row): turned through LDS so that the epilogue
+  // reads and writes whole rows. A wave reads its last K tile after the last barrier of the loops above,
+  // hence one more barrier before the rings are overwritten.
+  __syncthreads();
   OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * kD;
-  if (qrow < p.Sq) {
-    OutT* dst = dqh + qrow * q_row_stride;
-#pragma unroll
-    for (int o = 0; o < DB; ++o)
-#pragma unroll
-      for (int b4 = 0; b4 < 4; ++b4)
-        store4<OutT>(dst + 32 * o + 8 * b4 + 4 * g, acc[o][4 * b4] * p.scale, acc[o][4 * b4 + 1] * p.scale,
-                     acc[o][4 * b4 + 2] * p.scale, acc[o][4 * b4 + 3] * p.scale, p.accumulate != 0);
-  }
+  store_rows32_via_lds<OutT, DB>(smem + wave * kRowsViaLdsBytes<DB>, dqh + q_wave0 * q_row_stride, q_row_stride, p.Sq - q_wave0,
+                                 acc, p.scale, p.accumulate != 0, lane);
 }
 
 }  // namespace

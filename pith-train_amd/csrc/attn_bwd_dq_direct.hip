@@ -390,7 +390,12 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
 
   // ---- the late wave of a pair hands its partial dQ to the early wave (the tile ring is free: every
   // wave passed the barrier that ends the last interval)
-  constexpr int kExch = DB * 4 * 64 * 16;
+  // one area per wave pair; with 128 features it is used twice: for the late wave's partial dQ, then to turn the
+  // early wave's result tile (the 192-feature kernel keeps the direct stores: it has no register to spare, and any
+  // longer epilogue pushes spills into its main loop)
+  constexpr bool kTurn = DQK == 128;
+  constexpr int kExch = kTurn ? kRowsViaLdsBytes<DB> : DB * 4 * 64 * 16;
+  static_assert(kExch >= DB * 4 * 64 * 16 && 4 * kExch <= (int)sizeof(smem), "exchange area");
   char* const exch = smem + (wave & 3) * kExch;
   if constexpr (!HALF) {
     OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * DQK;
@@ -418,7 +423,19 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   if (late) return;
 
   OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * DQK;
-  if (qrow < p.Sq) {
+  if constexpr (kTurn) {
+    // the pair's dQ^T (a lane owns one query row) is turned through LDS - the same area, once the partner's values
+    // are in registers - so that the epilogue reads and writes whole rows
+#pragma unroll
+    for (int o = 0; o < DB; ++o)
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) {
+        const f32x4 v4 = *reinterpret_cast<const f32x4*>(exch + ((o * 4 + b4) * 64 + lane) * 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[o][4 * b4 + e] += v4[e];
+      }
+    store_rows32_via_lds<OutT, DB>(exch, dqh + q_wave0 * q_row_stride, q_row_stride, p.Sq - q_wave0, acc, p.scale, p.accumulate != 0, lane);
+  } else if (qrow < p.Sq) {
     OutT* dst = dqh + qrow * q_row_stride;
 #pragma unroll
     for (int o = 0; o < DB; ++o)

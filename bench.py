@@ -183,8 +183,8 @@ def handover_scratch_bytes(cfg, dev):
     most = 0
     for s in ring_schedule(cfg.rank, cfg.cp, cfg.s_local, LAYOUT):
         rows = slice(s.kv_rows[0], s.kv_rows[1])
-        need = hip.attn_bwd_ds_bytes(q[:, s.q_rows[0] : s.q_rows[1]], ks[s.kv_rank][:, rows], vs[s.kv_rank][:, rows], s.causal)
-        most = max(most, need if 0 < need <= hip.DS_BUFFER_LIMIT_BYTES else 0)
+        plan = hip.ds_plan(q[:, s.q_rows[0] : s.q_rows[1]], ks[s.kv_rank][:, rows], vs[s.kv_rank][:, rows], s.causal)
+        most = max(most, plan[1] if plan else 0)
     return most
 
 

@@ -163,7 +163,15 @@ int pith_attn_bwd_delta(const pith_attn_delta_args* args, pith_stream_t stream);
  * [B,Skv,Hkv,128] (the nope part and its gradient); dk_pe [B,Skv,64] (batch stride dk_pe_bs,
  * contiguous rows, dkv_dtype) receives the gradient of the shared rotary part, i.e. the sum over
  * heads of the last 64 features of the assembled key's gradient, added in head order through the
- * workspace (required then: pith_attn_bwd_dkdv_workspace_bytes). */
+ * workspace (required then: pith_attn_bwd_dkdv_workspace_bytes).
+ *
+ * A head range of wider tensors (q_row_heads / kv_row_heads != 0): the call works on Hq (Hkv)
+ * CONSECUTIVE heads of tensors whose rows hold q_row_heads (kv_row_heads) heads; q, dout, dq
+ * (k, v, dk, dv) point at the first head of the range, row strides are q_row_heads*D
+ * (kv_row_heads*D) elements, and lse / delta are addressed through their head stride as always.
+ * Results equal the corresponding heads of a call on all heads. This is how a caller bounds the
+ * dS hand-over buffer below: one kv head (and its query heads) at a time through one small buffer.
+ * Not available together with k_pe. */
 typedef struct {
   const void* q;
   const void* k;
@@ -190,6 +198,8 @@ typedef struct {
   int64_t dk_pe_bs;
   void* ds;                  /* optional dS hand-over buffer (see below), 256-byte aligned; may be NULL */
   int64_t ds_bytes;          /* its size */
+  int64_t q_row_heads;       /* heads per row of q, dout, dq (0 = Hq) */
+  int64_t kv_row_heads;      /* heads per row of k, v, dk, dv (0 = Hkv) */
 } pith_attn_bwd_args;
 
 int pith_attn_bwd_dkdv(const pith_attn_bwd_args* args, pith_stream_t stream);

@@ -16,6 +16,9 @@ struct BwdParams {
   void* dk;
   void* dv;
   int Sq, Skv, Hq, Hkv, group, B;
+  // heads per ROW of the query-side tensors (q, dout, dq) and of the key-side tensors (k, v, dk, dv): Hq / Hkv for
+  // tensors that hold exactly the heads of this call, larger when the call works on a head range of wider tensors
+  int HqT, HkvT;
   int tiles;  // query tiles (dQ kernel) or key tiles (dK/dV kernel) in the grid's x dimension
   int64_t q_bs, k_bs, v_bs, dout_bs, dq_bs, dk_bs, dv_bs, lse_bs, lse_hs;
   float kappa, scale;
@@ -86,6 +89,9 @@ __device__ __forceinline__ void store_rows32(OutT* block, int64_t row_stride, in
                                              float factor, bool accumulate, int c, int g) {
 #pragma clang fp contract(off)  // product rounded, then added: what accumulating into a separate tensor gives
   constexpr int kBatch = NB > 4 ? 4 : 8;  // accumulator elements per lane and batch: NB * kBatch old values in registers
+  // a block wholly beyond the last row (wave-uniform): `block` itself is out of range, so not even the clamped
+  // old-value loads may run
+  if (rows_valid <= 0) return;
 #pragma unroll
   for (int v0 = 0; v0 < 16; v0 += kBatch) {
     float old[kBatch][NB];

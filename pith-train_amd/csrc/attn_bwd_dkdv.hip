@@ -171,11 +171,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
   const int kv_pair0 = kv_wg0 + pair * 32;
   const int key = kv_pair0 + c;
 
-  const int64_t q_row_stride = (int64_t)p.Hq * DQK;
-  const int64_t do_row_stride = (int64_t)p.Hq * DV;
+  const int64_t q_row_stride = (int64_t)p.HqT * DQK;
+  const int64_t do_row_stride = (int64_t)p.HqT * DV;
   const int k_head = DQK;
-  const int64_t k_row_stride = (int64_t)p.Hkv * k_head;
-  const int64_t v_row_stride = (int64_t)p.Hkv * DV;
+  const int64_t k_row_stride = (int64_t)p.HkvT * k_head;
+  const int64_t v_row_stride = (int64_t)p.HkvT * DV;
 
   // stationary fragments: K rows for wave A, V rows for wave B
   bf16x8 stat[NSTAT];
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
     const int64_t row_stride = role_b ? k_row_stride : v_row_stride;
     if (p.split > 1) {
       float* ws = (role_b ? p.ws_dk : p.ws_dv) +
-                  (((int64_t)part * p.B + b) * p.Skv + key) * row_stride + (int64_t)hk * d;
+                  (((int64_t)part * p.B + b) * p.Skv + key) * ((int64_t)p.Hkv * d) + (int64_t)hk * d;  // partials are packed
 #pragma unroll
       for (int o = 0; o < NACC; ++o)
         if (o < nblk)
@@ -277,6 +277,7 @@ struct ReduceParams {
   const float* ws[2];
   void* out[2];
   int64_t part_stride[2], row_elems[2], out_bs[2], n4[2];
+  int64_t out_row_elems[2];  // elements between consecutive rows of `out` (>= row_elems: a head range of a wider tensor)
   int64_t rows_per_batch;
   int parts, accumulate;
 };
@@ -293,7 +294,9 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(ReduceParams r) {
     f32x4 s = *reinterpret_cast<const f32x4*>(ws + e);
     for (int pidx = 1; pidx < r.parts; ++pidx) s += *reinterpret_cast<const f32x4*>(ws + pidx * part_stride + e);
     const int64_t bb = e / per_batch;
-    OutT* dst = out + bb * r.out_bs[t] + (e - bb * per_batch);
+    const int64_t in_batch = e - bb * per_batch;
+    const int64_t row = in_batch / r.row_elems[t];
+    OutT* dst = out + bb * r.out_bs[t] + row * r.out_row_elems[t] + (in_batch - row * r.row_elems[t]);
     store4<OutT>(dst, s[0], s[1], s[2], s[3], r.accumulate != 0);
   }
 }
@@ -341,13 +344,13 @@ void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
   }
   if (p.k_pe) {  // dk_pe (+)= sum over heads, in head order
     ReduceParams r;
-    r.row_elems[0] = 64;
+    r.row_elems[0] = r.out_row_elems[0] = 64;
     r.part_stride[0] = a->B * a->Skv * 64;
     r.n4[0] = r.part_stride[0] / 4;
     r.ws[0] = p.ws_dkpe;
     r.out[0] = a->dk_pe;
     r.out_bs[0] = a->dk_pe_bs;
-    r.row_elems[1] = r.part_stride[1] = r.n4[1] = r.out_bs[1] = 0;
+    r.row_elems[1] = r.out_row_elems[1] = r.part_stride[1] = r.n4[1] = r.out_bs[1] = 0;
     r.ws[1] = nullptr;
     r.out[1] = nullptr;
     r.rows_per_batch = a->Skv;
@@ -364,6 +367,7 @@ void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
     for (int which = 0; which < 2; ++which) {
       const int64_t d = which == 0 ? a->Dqk : a->Dv;
       r.row_elems[which] = a->Hkv * d;
+      r.out_row_elems[which] = p.HkvT * d;
       r.part_stride[which] = a->B * a->Skv * r.row_elems[which];
       r.n4[which] = r.part_stride[which] / 4;
       r.ws[which] = which == 0 ? p.ws_dk : p.ws_dv;

@@ -36,6 +36,12 @@ constexpr int kStat = 2 * kBM * 4;               // lse[64], delta[64]
 constexpr int kStage = 2 * kTile + kStat;        // Q tile, dO tile, stats
 constexpr int kExchPair = kBM * 32 * 4;          // one 64 x 32 fp32 P tile
 constexpr int kSmem = kStages * kStage + 4 * kExchPair;
+// dS hand-over: vector-memory stores a B wave issues per interval (one 16-byte store per lane and 16-row step of
+// the 64-row tile). The wait that ends an interval lets exactly this many operations stay in flight, which is
+// right only while they are the LAST vector-memory operations the wave issued (tests/test_cabi.py checks that on
+// the compiler's output: loads first, then these stores, no spill traffic in the loop).
+constexpr int kDsStoresPerInterval = kBM / 16;
+static_assert(kDsStoresPerInterval == 4, "make_ds stores frag[0..3]; the vmcnt immediate below has a 4-bit low field");
 
 // Position of a query tile in the stream of (query head, tile) pairs a workgroup visits.
 struct TileCursor {
@@ -81,8 +87,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   const int kv_pair0 = kv_wg0 + pair * 32;
   const int key = kv_pair0 + c;
 
-  const int q_row_bytes = p.Hq * kD * 2;  // Q and dO rows
-  const int64_t kv_row_stride = (int64_t)p.Hkv * kD;
+  const int q_row_bytes = p.HqT * kD * 2;  // Q and dO rows
+  const int64_t kv_row_stride = (int64_t)p.HkvT * kD;
 
   // Query tiles to visit: all of them, or from the diagonal down under the causal mask.
   const int m_end = (p.Sq + kBM - 1) / kBM;
@@ -305,7 +311,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
       int off = (g << 9) + ((c ^ (g << 3)) << 4);  // recomputed per tile: no register is held across the interval
       asm volatile("" : "+v"(off));
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < kDsStoresPerInterval; ++j)
         __builtin_nontemporal_store(frag[j], reinterpret_cast<bf16x8*>(img + j * 1024 + (off ^ ((j & 1) << 6))));
     }
   };
@@ -326,7 +332,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
       // the tile requested in this interval has landed. Vector memory operations complete in issue
       // order, and where wave B issued its four dS stores after the request (every interval but the
       // first) they may stay in flight.
-      if (ROLE_B && EMIT_DS && stored) __builtin_amdgcn_s_waitcnt(0x0F74);
+      if (ROLE_B && EMIT_DS && stored) __builtin_amdgcn_s_waitcnt(0x0F70 | kDsStoresPerInterval);
       else __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
       done = cur;
@@ -388,7 +394,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   // ---- epilogue: wave A stores dV, wave B stores dK, for key row `key`, features 32*o + 8*b4 + 4*g ..+3
   if (key < p.Skv) {
     if (p.split > 1) {
-      float* ws = (role_b ? p.ws_dk : p.ws_dv) + (((int64_t)part * p.B + b) * p.Skv + key) * kv_row_stride + (int64_t)hk * kD;
+      // the partials are packed: exactly the Hkv heads of this call per row
+      float* ws = (role_b ? p.ws_dk : p.ws_dv) + (((int64_t)part * p.B + b) * p.Skv + key) * ((int64_t)p.Hkv * kD) + (int64_t)hk * kD;
 #pragma unroll
       for (int o = 0; o < DB; ++o)
 #pragma unroll

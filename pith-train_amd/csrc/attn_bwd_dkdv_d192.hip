@@ -112,11 +112,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
   const int kv_pair0 = kv_wg0 + pair * 32;
   const int key = kv_pair0 + c;
 
-  const int q_row_bytes = p.Hq * kDQ * 2, do_row_bytes = p.Hq * kDV * 2;
+  const int q_row_bytes = p.HqT * kDQ * 2, do_row_bytes = p.HqT * kDV * 2;
   const bool two_part = p.k_pe != nullptr;
   const int k_head = two_part ? 128 : kDQ;
-  const int64_t k_row_stride = (int64_t)p.Hkv * k_head;
-  const int64_t v_row_stride = (int64_t)p.Hkv * kDV;
+  const int64_t k_row_stride = (int64_t)p.HkvT * k_head;
+  const int64_t v_row_stride = (int64_t)p.HkvT * kDV;
 
   // Query tiles to visit: all of them, or from the diagonal down under the causal mask.
   const int m_end = (p.Sq + kBM - 1) / kBM;
@@ -425,7 +425,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
                         acc[o][4 * b4 + 3] * f, false);
     }
     if (p.split > 1) {
-      float* ws = (role_b ? p.ws_dk : p.ws_dv) + (((int64_t)part * p.B + b) * p.Skv + key) * row_stride + (int64_t)hk * d;
+      // the partials are packed: exactly the Hkv heads of this call per row
+      float* ws = (role_b ? p.ws_dk : p.ws_dv) + (((int64_t)part * p.B + b) * p.Skv + key) * ((int64_t)p.Hkv * d) + (int64_t)hk * d;
 #pragma unroll
       for (int o = 0; o < DB; ++o)
         if (o < nblk)

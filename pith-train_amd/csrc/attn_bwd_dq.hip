@@ -37,10 +37,10 @@ __global__ __launch_bounds__(WAVES * 64) void attn_bwd_dq_kernel(BwdParams p) {
   const int m0 = m_tile * BM;
   const int q_wave0 = m0 + wave * ROWS_WAVE;
 
-  const int64_t q_row_stride = (int64_t)p.Hq * DQK;
-  const int64_t do_row_stride = (int64_t)p.Hq * DV;
-  const int64_t k_row_stride = (int64_t)p.Hkv * DQK;
-  const int64_t v_row_stride = (int64_t)p.Hkv * DV;
+  const int64_t q_row_stride = (int64_t)p.HqT * DQK;
+  const int64_t do_row_stride = (int64_t)p.HqT * DV;
+  const int64_t k_row_stride = (int64_t)p.HkvT * DQK;
+  const int64_t v_row_stride = (int64_t)p.HkvT * DV;
   const __bf16* qh = p.q + b * p.q_bs + (int64_t)h * DQK;
   const __bf16* doh = p.dout + b * p.dout_bs + (int64_t)h * DV;
   const __bf16* kh = p.k + b * p.k_bs + (int64_t)hk * DQK;
@@ -244,6 +244,12 @@ int validate_bwd(const pith_attn_bwd_args* a, const char* who, bool need_dq, boo
                 (long long)a->B, (long long)a->Sq, (long long)a->Skv, (long long)a->Hq, (long long)a->Hkv);
   if (a->Hq % a->Hkv != 0)
     return fail(PITH_ERR_BAD_SHAPE, "%s: Hq=%lld is not a multiple of Hkv=%lld", who, (long long)a->Hq, (long long)a->Hkv);
+  if ((a->q_row_heads && (a->q_row_heads < a->Hq || a->q_row_heads > 65535)) ||
+      (a->kv_row_heads && (a->kv_row_heads < a->Hkv || a->kv_row_heads > 65535)))
+    return fail(PITH_ERR_BAD_SHAPE, "%s: q_row_heads=%lld / kv_row_heads=%lld must be 0 or at least Hq=%lld / Hkv=%lld", who,
+                (long long)a->q_row_heads, (long long)a->kv_row_heads, (long long)a->Hq, (long long)a->Hkv);
+  if (a->k_pe && (a->q_row_heads > a->Hq || a->kv_row_heads > a->Hkv))
+    return fail(PITH_ERR_UNSUPPORTED, "%s: keys in two parts cannot be combined with a head range of wider tensors", who);
   if (a->causal && a->Sq != a->Skv)
     return fail(PITH_ERR_UNSUPPORTED, "%s: causal needs Sq == Skv (got %lld, %lld)", who, (long long)a->Sq, (long long)a->Skv);
   if (a->Sq > (1 << 24) || a->Skv > (1 << 24) || a->Hq > 65535 || a->B > 65535 ||
@@ -279,6 +285,8 @@ BwdParams make_bwd_params(const pith_attn_bwd_args* a) {
   p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.dout = (const __bf16*)a->dout;
   p.lse = a->lse; p.delta = a->delta; p.dq = a->dq; p.dk = a->dk; p.dv = a->dv;
   p.Sq = (int)a->Sq; p.Skv = (int)a->Skv; p.Hq = (int)a->Hq; p.Hkv = (int)a->Hkv; p.group = (int)(a->Hq / a->Hkv); p.B = (int)a->B;
+  p.HqT = (int)(a->q_row_heads ? a->q_row_heads : a->Hq);
+  p.HkvT = (int)(a->kv_row_heads ? a->kv_row_heads : a->Hkv);
   p.tiles = 0;
   p.q_bs = a->q_bs; p.k_bs = a->k_bs; p.v_bs = a->v_bs; p.dout_bs = a->dout_bs;
   p.dq_bs = a->dq_bs; p.dk_bs = a->dk_bs; p.dv_bs = a->dv_bs; p.lse_bs = a->lse_bs; p.lse_hs = a->lse_hs;

@@ -48,8 +48,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
   const int q_wave0 = m0 + wave * 32;
   const int qrow = q_wave0 + c;
 
-  const int64_t q_row_stride = (int64_t)p.Hq * kD;
-  const int kv_row_bytes = p.Hkv * kD * 2;
+  const int64_t q_row_stride = (int64_t)p.HqT * kD;
+  const int kv_row_bytes = p.HkvT * kD * 2;
   const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * kD);
   const char* vh = reinterpret_cast<const char*>(p.v + b * p.v_bs + (int64_t)hk * kD);
 

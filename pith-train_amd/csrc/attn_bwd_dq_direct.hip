@@ -76,12 +76,12 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   const int q_wave0 = m0 + (HALF ? (wave & 3) : wave) * 32;
   const int qrow = q_wave0 + c;
 
-  const int64_t q_row_stride = (int64_t)p.Hq * DQK;
-  const int64_t do_row_stride = (int64_t)p.Hq * kDv;
+  const int64_t q_row_stride = (int64_t)p.HqT * DQK;
+  const int64_t do_row_stride = (int64_t)p.HqT * kDv;
   // keys in two parts: K rows hold 128 features per head, the last 64 come from k_pe (no head offset)
   const bool two_part = DQK == 192 && p.k_pe != nullptr;
   const int k_head_elems = two_part ? 128 : DQK;
-  const int k_row_bytes = p.Hkv * k_head_elems * 2, v_row_bytes = p.Hkv * kDv * 2;
+  const int k_row_bytes = p.HkvT * k_head_elems * 2, v_row_bytes = p.HkvT * kDv * 2;
   const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * k_head_elems);
   const char* kx = two_part ? reinterpret_cast<const char*>(p.k_pe + b * p.k_pe_bs) : kh;  // source of features 128..
   const int kx_row_bytes = two_part ? (int)p.k_pe_rs * 2 : k_row_bytes;

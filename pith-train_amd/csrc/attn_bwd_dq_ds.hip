@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
   const int m0 = m_tile * kBM;
   const int q_wave0 = m0 + wave * QW;
 
-  const int kv_row_bytes = p.Hkv * DQK * 2;
+  const int kv_row_bytes = p.HkvT * DQK * 2;
   const char* kh = reinterpret_cast<const char*>(p.k + b * p.k_bs + (int64_t)hk * DQK);
 
   // key steps: all of them, or up to the diagonal; a wave whose query tile does not exist (ragged
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
 
   OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * DQK;
   const float sc = -p.scale;  // the images hold -dS (the writer forms delta - dP)
-  const int64_t row_stride = (int64_t)p.Hq * DQK;
+  const int64_t row_stride = (int64_t)p.HqT * DQK;
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb) {
     const int row0 = q_wave0 + 32 * rb;

@@ -296,8 +296,8 @@ __device__ __forceinline__ bf16x8 lds_read_transposed_at(const char* lo_addr, co
 // turned through LDS first, every instruction reads or writes whole rows (2 rows x 512 bytes of fp32 per
 // instruction at 128 features). `lds` is a wave-private area of kRowsViaLdsBytes<NB> bytes (the tile
 // rings are free by then: the caller has passed the barrier behind their last reader); `factor` is this
-// lane's (= this row's) scale; rows at or beyond rows_valid are not written. With `accumulate` all old
-// values are read before the first store.
+// lane's (= this row's) scale; rows at or beyond rows_valid are neither read nor written (rows_valid may be <= 0).
+// With `accumulate` all old values are read before the first store.
 template <int NB>
 constexpr int kRowsViaLdsBytes = 32 * (NB * 128 + 16);
 
@@ -308,6 +308,9 @@ __device__ __forceinline__ void store_rows32_via_lds(char* lds, OutT* block, int
   constexpr int kPitch = NB * 128 + 16;  // bytes; the 16 spread the 32 rows of a column over the banks
   constexpr int kPieces = NB * 8;        // 16-byte pieces (4 features) per row
   constexpr int kIters = 32 * kPieces / 64;
+  // a block that lies wholly beyond the last row (the same for the whole wave): nothing to store, and the
+  // clamped old-value loads below would start from `block`, which is itself out of range then
+  if (rows_valid <= 0) return;
   const int c = lane & 31, g = lane >> 5;
 #pragma unroll
   for (int o = 0; o < NB; ++o)

@@ -82,6 +82,7 @@ class AttnBwdArgs(Structure):
         ("k_pe", c_void_p), ("k_pe_bs", c_int64), ("k_pe_rs", c_int64),
         ("dk_pe", c_void_p), ("dk_pe_bs", c_int64),
         ("ds", c_void_p), ("ds_bytes", c_int64),
+        ("q_row_heads", c_int64), ("kv_row_heads", c_int64),
     ]  # fmt: skip
 
 
@@ -197,6 +198,17 @@ def bshd_batch_stride(t: torch.Tensor, what: str) -> int:
     return sb if B > 1 else S * H * D
 
 
+def bshd_head_range_strides(t: torch.Tensor, what: str):
+    """Like bshd_batch_stride for a tensor that may also be a range of consecutive heads of a wider
+    [B,S,H_total,D] tensor (t = wide[:, s0:s1, h0:h1]); returns (batch stride in elements, heads per row)."""
+    B, S, H, D = t.shape
+    sb, ss, sh, sd = t.stride()
+    row_heads = H if S == 1 else ss // D
+    ok = (D == 1 or sd == 1) and (H == 1 or sh == D) and (S == 1 or (ss % D == 0 and row_heads >= H))
+    assert ok, f"{what} is not contiguous"
+    return (sb if B > 1 else S * row_heads * D), row_heads
+
+
 def bhs_strides(t: torch.Tensor, what: str):
     """Checks that a [B,H,S] tensor has unit stride along S; returns (batch, head) strides."""
     B, H, S = t.shape
@@ -207,5 +219,5 @@ def bhs_strides(t: torch.Tensor, what: str):
 
 __all__ = [
     "lib", "check", "PithError", "CombineArgs", "AttnFwdArgs", "AttnDeltaArgs", "AttnBwdArgs", "NormRopeArgs", "MlaAssembleArgs", "DeviceInfo", "SYMBOLS",
-    "dtype_code", "current_stream", "require_device", "bshd_batch_stride", "bhs_strides", "byref",
+    "dtype_code", "current_stream", "require_device", "bshd_batch_stride", "bshd_head_range_strides", "bhs_strides", "byref",
 ]  # fmt: skip

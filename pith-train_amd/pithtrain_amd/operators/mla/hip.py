@@ -126,17 +126,22 @@ def _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe=None) -> _C
     if k_pe is not None:
         k_pe, kpe_bs, kpe_rs = _k_pe_strides(k, k_pe)
         kpe_ptr = k_pe.data_ptr()
+    # q / dout (and k / v) may be the same range of consecutive heads of wider tensors
+    (q_bs, q_rh), (dout_bs, do_rh) = _C.bshd_head_range_strides(q, "q"), _C.bshd_head_range_strides(dout, "dout")
+    (k_bs, k_rh), (v_bs, v_rh) = _C.bshd_head_range_strides(k, "k"), _C.bshd_head_range_strides(v, "v")
+    assert q_rh == do_rh and k_rh == v_rh, "q / dout (k / v) must be the same head range of equally wide tensors"
+    assert k_pe is None or (q_rh == hq and k_rh == hkv), "keys in two parts cannot be combined with a head range"
     return _C.AttnBwdArgs(
         k_pe=kpe_ptr, k_pe_bs=kpe_bs, k_pe_rs=kpe_rs, dk_pe=None, dk_pe_bs=0,
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), dout=dout.data_ptr(),
         lse=lse.data_ptr(), delta=delta.data_ptr(), dq=None, dk=None, dv=None,
         B=b, Sq=sq, Skv=skv, Hq=hq, Hkv=hkv, Dqk=d_q, Dv=d_v,
-        q_bs=_C.bshd_batch_stride(q, "q"), k_bs=_C.bshd_batch_stride(k, "k"),
-        v_bs=_C.bshd_batch_stride(v, "v"), dout_bs=_C.bshd_batch_stride(dout, "dout"),
+        q_bs=q_bs, k_bs=k_bs, v_bs=v_bs, dout_bs=dout_bs,
         dq_bs=0, dk_bs=0, dv_bs=0, lse_bs=lse_bs, lse_hs=lse_hs,
         scale=float(softmax_scale), causal=int(bool(causal)),
         dq_dtype=_C.PITH_BF16, dkv_dtype=_C.PITH_BF16, accumulate_dq=0, accumulate_dkv=0,
         workspace=None, workspace_bytes=0, ds=None, ds_bytes=0,
+        q_row_heads=q_rh, kv_row_heads=k_rh,
     )  # fmt: skip
 
 
@@ -157,11 +162,15 @@ def _set_ds(args, ds: torch.Tensor, like: torch.Tensor) -> None:
     args.ds, args.ds_bytes = ds.data_ptr(), ds.numel()
 
 
-# Above this size the hand-over buffer is not worth its memory: the two backward calls recompute.
-# The hand-over makes the backward 3-6 % faster at the price of Sq*Skv*Hq*B*2 bytes of scratch while the two
-# kernels run (2 GiB per ring step at 32 heads and 8192 x 4096 rows, 16 GiB at 64 heads and 16384 x 8192; a
-# causal pair needs half of the full rectangle plus its diagonal blocks: 16.1 GiB at 64 heads and 16384 rows).
-DS_BUFFER_LIMIT_BYTES = int(float(os.environ.get("PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB", "17")) * (1 << 30))
+# The dS hand-over (head dims 128/128) makes the backward of a chunk pair 3-6 % faster at the price of a
+# transient buffer of Sq*Skv*Hq*B*2 bytes while the pair's two kernels run (about half under the causal mask).
+# Policy: the buffer never exceeds DS_BUFFER_LIMIT_BYTES nor DS_BUFFER_FREE_FRACTION of the device memory that is
+# free right now; a chunk pair that needs more is processed one group of kv heads (with their query heads) after
+# the other through one buffer of the bounded size; when not even one kv head fits, or the allocation fails, the
+# two kernels recompute the scores as the reference's do (pithtrain/operators/mla/triton.py:130-266), which needs
+# no scratch at all.
+DS_BUFFER_LIMIT_BYTES = int(float(os.environ.get("PITHTRAIN_AMD_DS_BUFFER_LIMIT_GB", "4")) * (1 << 30))
+DS_BUFFER_FREE_FRACTION = 0.5
 _DS_ROWS_PER_WORKGROUP = 512  # query rows a workgroup of the dS-reading dQ kernel owns
 _compute_units = {}
 
@@ -175,18 +184,81 @@ def _device_compute_units(device: torch.device) -> int:
     return _compute_units[idx]
 
 
-def ds_buffer(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool = False):
-    """A dS hand-over buffer for one chunk pair from torch's caching allocator, or None when the
-    shape has no hand-over path, the buffer would exceed DS_BUFFER_LIMIT_BYTES, or the dS-reading dQ
-    kernel would have fewer workgroups than the device has compute units (the recomputing kernels
-    use smaller workgroups and then win)."""
+def _ds_budget_bytes(device: torch.device) -> int:
+    """What a hand-over buffer may take right now: the configured limit, and at most a fraction of the
+    memory that is free on the device or cached (unused) by torch's allocator."""
+    free, _ = torch.cuda.mem_get_info(device)
+    cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
+    return min(DS_BUFFER_LIMIT_BYTES, int((free + max(cached, 0)) * DS_BUFFER_FREE_FRACTION))
+
+
+def ds_plan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool = False):
+    """How the backward of one chunk pair uses the dS hand-over: (kv heads per slab, bytes of the buffer),
+    or None when both kernels should recompute (no hand-over path for these head dims, the dS-reading dQ
+    kernel would have fewer workgroups than the device has compute units, or not even one kv head fits the
+    budget)."""
     need = attn_bwd_ds_bytes(q, k, v, causal)
-    if need == 0 or need > DS_BUFFER_LIMIT_BYTES:
+    if need == 0:
         return None
     b, sq, hq, _ = q.shape
-    if -(-sq // _DS_ROWS_PER_WORKGROUP) * hq * b < _device_compute_units(q.device):
+    hkv = k.shape[2]
+    budget = _ds_budget_bytes(q.device)
+    per_kv_head = need // hkv
+    heads = hkv
+    while heads > 1 and per_kv_head * heads > budget:
+        heads -= 1
+        while hkv % heads:
+            heads -= 1
+    if per_kv_head * heads > budget:
         return None
-    return torch.empty(need, dtype=torch.uint8, device=q.device)
+    if -(-sq // _DS_ROWS_PER_WORKGROUP) * (hq // hkv) * heads * b < _device_compute_units(q.device):
+        return None
+    return heads, per_kv_head * heads
+
+
+def ds_buffer(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool = False):
+    """A dS hand-over buffer for the WHOLE chunk pair from torch's caching allocator, or None when
+    ds_plan says the pair should recompute or be processed in slabs, or when the allocation fails."""
+    plan = ds_plan(q, k, v, causal)
+    if plan is None or plan[0] != k.shape[2]:
+        return None
+    return _try_alloc(plan[1], q.device)
+
+
+def _try_alloc(nbytes: int, device: torch.device):
+    try:
+        return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    except torch.cuda.OutOfMemoryError:
+        return None
+
+
+def attn_bwd_pair_into(
+    q, k, v, dout, lse, delta, dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor, softmax_scale: float, causal: bool,
+    accumulate_dq: bool = False, accumulate_dkv: bool = False, k_pe: torch.Tensor = None, dk_pe: torch.Tensor = None,
+    handover: bool = True,
+) -> int:  # fmt: skip
+    """Both backward calls of one chunk pair: dk, dv, then dq (see attn_bwd_dkdv_into / attn_bwd_dq_into).
+    The dS hand-over between them is decided here (ds_plan), so a buffer can never reach the dQ call without
+    the dK/dV call that fills it. Returns the bytes of hand-over scratch used (0: both kernels recomputed)."""
+    plan = ds_plan(q, k, v, causal) if handover and k_pe is None else None
+    buf = _try_alloc(plan[1], q.device) if plan is not None else None
+    hkv = k.shape[2]
+    if buf is None or plan[0] == hkv:
+        attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, softmax_scale, causal, accumulate=accumulate_dkv,
+                           k_pe=k_pe, dk_pe=dk_pe, ds=buf)  # fmt: skip
+        attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, softmax_scale, causal, accumulate=accumulate_dq, k_pe=k_pe, ds=buf)
+        return 0 if buf is None else buf.numel()
+    # one group of kv heads after the other, each with its query heads, through the same buffer (the
+    # kernels of successive slabs are ordered by the stream)
+    group = q.shape[2] // hkv
+    for h0 in range(0, hkv, plan[0]):
+        kv_h, q_h = slice(h0, h0 + plan[0]), slice(h0 * group, (h0 + plan[0]) * group)
+        qs, ds_, ls, dl = q[:, :, q_h], dout[:, :, q_h], lse[:, q_h], delta[:, q_h]
+        attn_bwd_dkdv_into(qs, k[:, :, kv_h], v[:, :, kv_h], ds_, ls, dl, dk[:, :, kv_h], dv[:, :, kv_h],
+                           softmax_scale, causal, accumulate=accumulate_dkv, ds=buf)  # fmt: skip
+        attn_bwd_dq_into(qs, k[:, :, kv_h], v[:, :, kv_h], ds_, ls, dl, dq[:, :, q_h], softmax_scale, causal,
+                         accumulate=accumulate_dq, ds=buf)  # fmt: skip
+    return buf.numel()
 
 
 def attn_bwd_dkdv_into(
@@ -211,7 +283,8 @@ def attn_bwd_dkdv_into(
         args.dk_pe = dk_pe.data_ptr()
         args.dk_pe_bs = dk_pe.stride(0) if b > 1 else s * 64
     args.dk, args.dv = dk.data_ptr(), dv.data_ptr()
-    args.dk_bs, args.dv_bs = _C.bshd_batch_stride(dk, "dk"), _C.bshd_batch_stride(dv, "dv")
+    (args.dk_bs, dk_rh), (args.dv_bs, dv_rh) = _C.bshd_head_range_strides(dk, "dk"), _C.bshd_head_range_strides(dv, "dv")
+    assert dk_rh == dv_rh == args.kv_row_heads, "dk / dv must be laid out like k / v"
     args.dkv_dtype = _C.dtype_code(dk)
     args.accumulate_dkv = int(bool(accumulate))
     # Scratch for the head-split partial sums; the caching allocator makes this a pointer bump,
@@ -236,7 +309,8 @@ def attn_bwd_dq_into(
     _C.require_device(q, dq)
     assert dq.shape == q.shape, "dq must match q"
     args.dq = dq.data_ptr()
-    args.dq_bs = _C.bshd_batch_stride(dq, "dq")
+    args.dq_bs, dq_rh = _C.bshd_head_range_strides(dq, "dq")
+    assert dq_rh == args.q_row_heads, "dq must be laid out like q"
     args.dq_dtype = _C.dtype_code(dq)
     args.accumulate_dq = int(bool(accumulate))
     _C.check(_C.lib().pith_attn_bwd_dq(_C.byref(args), _C.current_stream(q)))
@@ -315,9 +389,7 @@ def _attn_bwd_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Ten
     q, k, v, o, dout = q.contiguous(), k.contiguous(), v.contiguous(), o.contiguous(), dout.contiguous()
     delta = _mla_bwd_preprocess(o, dout)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    ds = ds_buffer(q, k, v, causal)
-    attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, softmax_scale, causal, ds=ds)
-    attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, softmax_scale, causal, ds=ds)
+    attn_bwd_pair_into(q, k, v, dout, lse, delta, dq, dk, dv, softmax_scale, causal)
     return dq, dk, dv
 
 
@@ -384,5 +456,6 @@ class MLA(nn.Module):
 
 __all__ = [
     "MLA", "attention_func", "_mla_fwd", "_mla_bwd_preprocess", "_mla_bwd_dk_dv", "_mla_bwd_dq",
-    "attn_fwd_into", "attn_bwd_delta_into", "attn_bwd_dkdv_into", "attn_bwd_dq_into",
+    "attn_fwd_into", "attn_bwd_delta_into", "attn_bwd_dkdv_into", "attn_bwd_dq_into", "attn_bwd_pair_into",
+    "ds_plan", "ds_buffer",
 ]  # fmt: skip

@@ -62,14 +62,20 @@ class RingAttentionDistributedFunc(torch.autograd.Function):
     measure it on). The reference waits for each exchange before it computes (standard.py:95-98);
     the data each step sees is the same.
 
-    k_pe (optional, last argument): keys in two parts. k is then the 128-feature k_nope and k_pe
+    The first seven arguments are the reference's (standard.py:73, mla.py:47) and may be all that is
+    passed; the backward then returns the reference's seven gradients (standard.py:189, mla.py:149).
+    Up to three more may follow: layout ("contiguous"), rerotate (False) and k_pe (None).
+
+    k_pe: keys in two parts. k is then the 128-feature k_nope and k_pe
     [B, S_l, 64] the rotary part shared by all heads; both travel around the ring (16.5 MB instead
     of the assembled key's 24 MB per chunk of 4096 tokens and 16 heads), and the backward returns
     gradients for both."""
 
     @staticmethod
-    def forward(ctx, q, k, v, softmax_scale, cp_rank, cp_size, global_ranks, layout="contiguous", rerotate=False,
-                k_pe=None):  # fmt: skip
+    def forward(ctx, q, k, v, softmax_scale, cp_rank, cp_size, global_ranks, *extra):
+        assert len(extra) <= 3, "at most layout, rerotate and k_pe may follow the reference's seven arguments"
+        layout, rerotate, k_pe = (*extra, *("contiguous", False, None)[len(extra) :])
+        ctx.n_extra = len(extra)
         assert k.is_contiguous() and v.is_contiguous(), "ring attention k or v is not contiguous"
         order = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
         steps = {st.kv_rank: st for st in order}
@@ -116,7 +122,7 @@ class RingAttentionDistributedFunc(torch.autograd.Function):
             grads = _backward_rerotating(dout, q, out, lse, chunks[cp_rank], softmax_scale, cp_rank, cp_size,
                                          global_ranks, layout)  # fmt: skip
             dk_pe = (grads[3].unsqueeze(2) if ctx.k_pe_4d else grads[3]) if ctx.two_part else None
-            return grads[0], grads[1], grads[2], None, None, None, None, None, None, dk_pe
+            return (grads[0], grads[1], grads[2], None, None, None, None, *(None, None, dk_pe)[: ctx.n_extra])
         order = ring_schedule(cp_rank, cp_size, q.shape[1], layout)
         by_rank = {st.kv_rank: st for st in order}
         bwd = RingBackward(dout, q, out, lse, softmax_scale, order)
@@ -157,7 +163,8 @@ class RingAttentionDistributedFunc(torch.autograd.Function):
                 for mine, theirs in zip(local, recv):
                     mine += theirs
         dk_pe = (local[2].unsqueeze(2) if ctx.k_pe_4d else local[2]) if ctx.two_part else None
-        return dq, local[0], local[1], None, None, None, None, None, None, dk_pe
+        # one gradient per forward argument: the reference's seven, then those of the optional ones passed
+        return (dq, local[0], local[1], None, None, None, None, *(None, None, dk_pe)[: ctx.n_extra])
 
 
 def _backward_rerotating(dout, q, out, lse, chunk, softmax_scale, cp_rank, cp_size, global_ranks, layout):

@@ -43,10 +43,8 @@ import torch
 from pithtrain_amd import _C
 from pithtrain_amd.operators.mla.hip import (
     attn_bwd_delta_into,
-    attn_bwd_dkdv_into,
-    attn_bwd_dq_into,
+    attn_bwd_pair_into,
     attn_fwd_into,
-    ds_buffer,
 )
 from pithtrain_amd.operators.ring_attention.combine import cast_f32_bf16_into, combine_into
 
@@ -223,6 +221,8 @@ class RingBackward:
         single = len(self.steps) == 1
         self.dq_acc = self.dq if single else torch.empty(q.shape, dtype=torch.float32, device=q.device)
         self.done = 0
+        self.handover = True  # False: every step's two kernels recompute the scores (no dS scratch)
+        self.scratch_bytes = 0  # largest dS hand-over buffer a step has used so far
 
     def run_step(self, st: RingStep, k_j: torch.Tensor, v_j: torch.Tensor, add_to=None, k_pe_j: torch.Tensor = None):
         """Returns (dk_j, dv_j), this rank's contribution to chunk st.kv_rank's gradients; with
@@ -253,15 +253,13 @@ class RingBackward:
         ks, vs = _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows)
         ls, dl = _lse_rows(self.lse, st.q_rows), _lse_rows(self.delta, st.q_rows)
         pes = _pe_rows(k_pe_j, st.kv_rows)
-        # The dK/dV kernel leaves its dS tiles in `hand` for the dQ kernel, which then skips the score
-        # recomputation (head dims 128/128; None otherwise: both kernels recompute).
-        hand = ds_buffer(qs, ks, vs, st.causal) if pes is None else None
-        attn_bwd_dkdv_into(qs, ks, vs, ds, ls, dl, _rows(dk_j, st.kv_rows), _rows(dv_j, st.kv_rows),
-                           self.scale, st.causal, accumulate=add_to is not None, k_pe=pes,
-                           dk_pe=_pe_rows(dk_pe_j, st.kv_rows), ds=hand)  # fmt: skip
-        # Step 0 covers every row and initialises the accumulator; later steps add to their rows.
-        attn_bwd_dq_into(qs, ks, vs, ds, ls, dl, _rows(self.dq_acc, st.q_rows), self.scale, st.causal,
-                         accumulate=self.done > 0, k_pe=pes, ds=hand)  # fmt: skip
+        # dK/dV, then dQ; the pair helper decides whether the dK/dV kernel leaves its dS tiles for the dQ
+        # kernel (head dims 128/128, bounded scratch) or both kernels recompute the scores.
+        # Step 0 covers every row and initialises the dQ accumulator; later steps add to their rows.
+        self.scratch_bytes = max(self.scratch_bytes, attn_bwd_pair_into(
+            qs, ks, vs, ds, ls, dl, _rows(self.dq_acc, st.q_rows), _rows(dk_j, st.kv_rows), _rows(dv_j, st.kv_rows),
+            self.scale, st.causal, accumulate_dq=self.done > 0, accumulate_dkv=add_to is not None, k_pe=pes,
+            dk_pe=_pe_rows(dk_pe_j, st.kv_rows), handover=self.handover))  # fmt: skip
         self.done += 1
         return (dk_j, dv_j) if k_pe_j is None else (dk_j, dv_j, dk_pe_j)
 

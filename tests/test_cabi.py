@@ -274,7 +274,24 @@ def test_ring_schedule_matches_oracle_schedule():
                 assert ours == R._steps(r, C, 64, layout)
 
 
-def test_m0_is_touched_only_by_the_direct_load_statements(tmp_path):
+_ASM_CACHE = {}
+
+
+def _kernel_asm(src, tmp_dir):
+    """gfx950 assembly of one kernel source (compiled once per test session)."""
+    from pithtrain_amd import build as B
+
+    if src not in _ASM_CACHE:
+        out = os.path.join(str(tmp_dir), src + ".s")
+        cmd = [B._hipcc(), *B.HIPCC_FLAGS, "-I", B.INCLUDE_DIR, "-I", B.SRC_DIR, "--cuda-device-only", "-S",
+               os.path.join(B.SRC_DIR, src), "-o", out]  # fmt: skip
+        subprocess.run(cmd, check=True, capture_output=True)
+        with open(out) as f:
+            _ASM_CACHE[src] = f.read()
+    return _ASM_CACHE[src]
+
+
+def test_m0_is_touched_only_by_the_direct_load_statements(tmp_path_factory):
     """csrc/attn_tiles.h sets M0 inside inline assembly (the LDS destination of global_load_lds), which
     the compiler cannot be told about. Compile every kernel source to gfx950 assembly and check that
     no instruction OUTSIDE the inline-assembly regions (;;#ASMSTART ... ;;#ASMEND) mentions M0, i.e. that the
@@ -283,13 +300,11 @@ def test_m0_is_touched_only_by_the_direct_load_statements(tmp_path):
 
     from pithtrain_amd import build as B
 
+    tmp = tmp_path_factory.getbasetemp()
+
     def offending(src):
-        out = tmp_path / (src + ".s")
-        cmd = [B._hipcc(), *B.HIPCC_FLAGS, "-I", B.INCLUDE_DIR, "-I", B.SRC_DIR, "--cuda-device-only", "-S",
-               os.path.join(B.SRC_DIR, src), "-o", str(out)]  # fmt: skip
-        subprocess.run(cmd, check=True, capture_output=True)
         bad, in_asm = [], False
-        for line in out.read_text().splitlines():
+        for line in _kernel_asm(src, tmp).splitlines():
             code = line.split(";")[0]
             if "#ASMSTART" in line:
                 in_asm = True
@@ -306,3 +321,38 @@ def test_m0_is_touched_only_by_the_direct_load_statements(tmp_path):
     with ThreadPoolExecutor(max_workers=8) as pool:
         bad = [b for res in pool.map(offending, users) for b in res]
     assert not bad, "compiler-generated M0 use next to inline M0 writes:\n" + "\n".join(bad[:10])
+
+
+def test_ds_storing_dkdv_kernel_waits_for_its_tile_loads_only(tmp_path_factory):
+    """The dK/dV kernel that also stores its dS tiles ends an interval with `s_waitcnt vmcnt(4)`: the tile
+    requests of the interval must have landed, its four dS stores may stay in flight. Vector memory operations
+    retire in issue order, so this is only right if, in the steady-state loop of the storing waves, every load is
+    issued before the first store, exactly four stores follow, and no register spill traffic (which counts in
+    vmcnt as well) sits in the loop. Checked on the compiler's output."""
+    from pithtrain_amd import build as B  # noqa: F401
+
+    text = _kernel_asm("attn_bwd_dkdv_d128.hip", tmp_path_factory.getbasetemp())
+    lines = text.splitlines()
+    waits = [i for i, l in enumerate(lines) if re.search(r"s_waitcnt vmcnt\(4\)\s*$", l) and "s_barrier" in lines[i + 1]]
+    assert len(waits) == 4, f"expected one steady-state wait per storing kernel variant (2 masks x 2 output types), got {len(waits)}"
+    for w in waits:
+        head = max(i for i in range(w) if "Inner Loop Header" in lines[i])
+        label = re.match(r"\.(LBB\d+_\d+):", lines[head]).group(1)
+        body = lines[head:w]
+        ops = [l.split()[0] for l in body if re.match(r"\s+(global_|scratch_|buffer_|flat_)", l)]
+        assert not [o for o in ops if o.startswith(("scratch_", "buffer_", "flat_"))], f"spill or foreign memory traffic in the loop: {ops}"
+        stores = [i for i, o in enumerate(ops) if o.startswith("global_store")]
+        assert len(stores) == 4, f"the loop must issue exactly the four dS stores, found {len(stores)}"
+        assert stores == list(range(len(ops) - 4, len(ops))), f"a load is issued after a store: {ops}"
+        assert any(o.startswith("global_load_lds") for o in ops[: stores[0]]), "the tile requests must precede the stores"
+        # blocks of the same loop that the compiler placed out of line (ragged-tile requests) hold loads only
+        end = next(i for i in range(w, len(lines)) if "s_endpgm" in lines[i])
+        in_loop_blocks = []
+        cur = None
+        for l in lines[w:end]:
+            m = re.match(r"\.(LBB\d+_\d+):(.*)", l)
+            if m:
+                cur = f"Header=B{label[2:]}" in m.group(2)
+            elif cur and re.match(r"\s+(global_store|scratch_)", l):
+                in_loop_blocks.append(l.strip())
+        assert not in_loop_blocks, f"stores or spills in out-of-line blocks of the loop: {in_loop_blocks}"

@@ -42,8 +42,11 @@ def _install_cpu_stand_ins():
         rdq, _, _ = R.chunk_bwd(q, full_key(k, k_pe), v, dout, lse.double(), delta.double(), scale, causal)
         dq.copy_(dq.double() + rdq if accumulate else rdq)
 
-    def ds_buffer(q, k, v, causal=False):  # no dS hand-over between the stand-ins
-        return None
+    def attn_bwd_pair_into(q, k, v, dout, lse, delta, dq, dk, dv, scale, causal, accumulate_dq=False,
+                           accumulate_dkv=False, k_pe=None, dk_pe=None, handover=True):  # fmt: skip
+        attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, scale, causal, accumulate_dkv, k_pe, dk_pe)
+        attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, scale, causal, accumulate_dq, k_pe)
+        return 0  # no dS hand-over between the stand-ins
 
     def combine_into(out1, lse1, out2, lse2, out, lse_out, base=0):
         o, l = R.combine_log2(out1.double(), lse1.double(), out2.double(), lse2.double())

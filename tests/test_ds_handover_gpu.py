@@ -132,17 +132,21 @@ def test_ring_share_uses_the_handover(gpu, layout, monkeypatch):
         out.backward(dos[rank].to(gpu))
         return q.grad, [t.grad for t in kc], [t.grad for t in vc]
 
-    calls = []
+    from pithtrain_amd.operators.mla import hip as H
+
+    used = []
+    real_plan = H.ds_plan
 
     def always(q, k, v, causal=False):  # the default policy would decline a share this small
-        calls.append(1)
-        return torch.empty(attn_bwd_ds_bytes(q, k, v, causal), dtype=torch.uint8, device=q.device)
+        used.append(1)
+        return k.shape[2], attn_bwd_ds_bytes(q, k, v, causal)
 
-    monkeypatch.setattr(L, "ds_buffer", always)
+    monkeypatch.setattr(H, "ds_plan", always)
     dq1, dk1, dv1 = run()
-    assert calls, "the ring backward did not ask for a hand-over buffer"
-    monkeypatch.setattr(L, "ds_buffer", lambda *a: None)
+    assert used, "the ring backward did not ask for a hand-over plan"
+    monkeypatch.setattr(H, "ds_plan", lambda *a: None)
     dq0, dk0, dv0 = run()
+    monkeypatch.setattr(H, "ds_plan", real_plan)
     for a, b in zip(dk0 + dv0, dk1 + dv1):
         assert (a is None and b is None) or torch.equal(a, b)
     assert norm_max_err(dq1.float().cpu(), dq0.float().cpu()) < 6e-3
@@ -151,21 +155,126 @@ def test_ring_share_uses_the_handover(gpu, layout, monkeypatch):
     check_bf16_result(dq1, dq_ref, "ring dQ", otol=1e-3)
 
 
+def _shaped(gpu, b, s, hq, hkv):
+    q = torch.empty(b, s, hq, 128, dtype=torch.bfloat16, device=gpu)
+    k = torch.empty(b, s, hkv, 128, dtype=torch.bfloat16, device=gpu)
+    return q, k, k
+
+
 def test_default_policy_of_the_buffer(gpu, monkeypatch):
-    """ds_buffer hands out a buffer only when it stays under the size limit and the dS-reading dQ kernel
-    would fill the device; otherwise the ring backward recomputes."""
+    """ds_plan takes the hand-over only when the dS-reading dQ kernel would fill the device, keeps the buffer
+    under the configured limit and under a fraction of the free memory by going through the kv heads in slabs,
+    and gives up (both kernels recompute) when not even one kv head fits."""
     from pithtrain_amd.operators.mla import hip as H
 
-    def shaped(b, s, hq, hkv):
-        q = torch.empty(b, s, hq, 128, dtype=torch.bfloat16, device=gpu)
-        k = torch.empty(b, s, hkv, 128, dtype=torch.bfloat16, device=gpu)
-        return q, k, k
-
-    assert ds_buffer(*shaped(1, 512, 8, 2)) is None  # 1 x 8 workgroups: too few
-    big = shaped(1, 4096, 32, 4)  # 8 x 32 workgroups, 1 GiB
+    assert H.DS_BUFFER_LIMIT_BYTES <= 4 << 30, "the default limit must stay modest"
+    assert H.ds_plan(*_shaped(gpu, 1, 512, 8, 2)) is None  # 1 x 8 workgroups: too few
+    big = _shaped(gpu, 1, 4096, 32, 4)  # 8 x 32 workgroups, 1 GiB
     assert attn_bwd_ds_bytes(*big) == 1 << 30
+    assert H.ds_plan(*big) == (4, 1 << 30)
     buf = ds_buffer(*big)
     assert buf is not None and buf.numel() == 1 << 30 and buf.data_ptr() % 256 == 0
     del buf
     monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (1 << 30) - 1)
-    assert ds_buffer(*big) is None
+    assert H.ds_plan(*big) == (2, 1 << 29) and ds_buffer(*big) is None  # two slabs of two kv heads
+    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (1 << 28) + 5)
+    assert H.ds_plan(*big) == (1, 1 << 28)
+    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (1 << 28) - 1)
+    assert H.ds_plan(*big) is None
+    # the 131072-token configuration (64 / 4 heads, 16384 x 8192 rows per ring step): one kv head at a time
+    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", 4 << 30)
+    q = torch.empty(1, dtype=torch.bfloat16, device=gpu).as_strided((1, 16384, 64, 128), (0, 0, 0, 0))
+    k = torch.empty(1, dtype=torch.bfloat16, device=gpu).as_strided((1, 8192, 4, 128), (0, 0, 0, 0))
+    assert H.ds_plan(q, k, k) == (1, 4 << 30)
+    # little free memory: the budget follows it
+    monkeypatch.setattr(H.torch.cuda, "mem_get_info", lambda dev=None: (1 << 29, 1 << 38))
+    monkeypatch.setattr(H.torch.cuda, "memory_reserved", lambda dev=None: 0)
+    monkeypatch.setattr(H.torch.cuda, "memory_allocated", lambda dev=None: 0)
+    assert H.ds_plan(*big) == (1, 1 << 28)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_slabs_of_kv_heads_equal_the_whole_call(gpu, causal, monkeypatch):
+    """attn_bwd_pair_into through a buffer that holds one or two kv heads at a time (head ranges of the full
+    tensors, passed in place) gives dK/dV bit for bit and dQ bit for bit what the whole-pair hand-over gives."""
+    from pithtrain_amd.operators.mla import hip as H
+
+    B, Sq, Hq, Hkv = 2, 1024, 16, 4
+    Skv = Sq if causal else 640
+    q, k, v, dout, scale = _inputs(B, Sq, Skv, Hq, Hkv, seed=11)
+    qd, kd, vd, dod = (t.to(gpu) for t in (q, k, v, dout))
+    o, lse = _mla_fwd(qd, kd, vd, scale, causal)
+    delta = _mla_bwd_preprocess(o, dod)
+    need = attn_bwd_ds_bytes(qd, kd, vd, causal)
+    results = []
+    for heads in (4, 2, 1):
+        monkeypatch.setattr(H, "ds_plan", lambda *a, heads=heads: (heads, need // Hkv * heads))
+        dq = torch.full(qd.shape, 0.25, dtype=torch.float32, device=gpu)
+        dk, dv = torch.empty_like(kd), torch.empty_like(vd)
+        used = H.attn_bwd_pair_into(qd, kd, vd, dod, lse, delta, dq, dk, dv, scale, causal, accumulate_dq=True)
+        assert used == need // Hkv * heads
+        results.append((dq, dk, dv))
+    for dq, dk, dv in results[1:]:
+        assert torch.equal(dq, results[0][0]) and torch.equal(dk, results[0][1]) and torch.equal(dv, results[0][2])
+    rdq, rdk, rdv = R.chunk_bwd(q, k, v, dout, lse.double().cpu(), delta.double().cpu(), scale, causal)
+    check_bf16_result(results[2][0] - 0.25, rdq, "slab dQ", otol=1e-3)
+    check_bf16_result(results[2][1], rdk, "slab dK", otol=1e-3)
+    check_bf16_result(results[2][2], rdv, "slab dV", otol=1e-3)
+
+
+def test_head_range_calls_without_handover(gpu):
+    """The recomputing kernels accept a head range of wider tensors too (all three head-dim families)."""
+    for d_q, d_v in ((128, 128), (192, 128), (64, 64)):
+        B, S, Hq, Hkv = 1, 320, 8, 4
+        g = torch.Generator().manual_seed(5)
+        q = (torch.randn(B, S, Hq, d_q, generator=g) * d_q**-0.5).to(torch.bfloat16).to(gpu)
+        k = (torch.randn(B, S, Hkv, d_q, generator=g) * d_q**-0.5).to(torch.bfloat16).to(gpu)
+        v = torch.randn(B, S, Hkv, d_v, generator=g).to(torch.bfloat16).to(gpu)
+        dout = torch.randn(B, S, Hq, d_v, generator=g).to(torch.bfloat16).to(gpu)
+        scale = d_q**-0.5
+        o, lse = _mla_fwd(q, k, v, scale, True)
+        delta = _mla_bwd_preprocess(o, dout)
+        dq0, dk0, dv0 = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        from pithtrain_amd.operators.mla import hip as H_
+
+        H_.attn_bwd_pair_into(q, k, v, dout, lse, delta, dq0, dk0, dv0, scale, True, handover=False)
+        dq1, dk1, dv1 = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+        for h0 in range(0, Hkv, 2):
+            kv_h, q_h = slice(h0, h0 + 2), slice(2 * h0, 2 * h0 + 4)
+            H_.attn_bwd_pair_into(q[:, :, q_h], k[:, :, kv_h], v[:, :, kv_h], dout[:, :, q_h], lse[:, q_h], delta[:, q_h],
+                                  dq1[:, :, q_h], dk1[:, :, kv_h], dv1[:, :, kv_h], scale, True, handover=False)  # fmt: skip
+        assert torch.equal(dq0, dq1) and torch.equal(dk0, dk1) and torch.equal(dv0, dv1), (d_q, d_v)
+
+
+def test_allocation_failure_falls_back_to_recomputation(gpu, monkeypatch):
+    """When the hand-over buffer cannot be allocated the pair recomputes: dK/dV bit-identical to the hand-over
+    path (the dK/dV kernel's arithmetic does not depend on the stores), dQ within oracle parity."""
+    from pithtrain_amd.operators.mla import hip as H
+
+    B, Sq, Skv, Hq, Hkv = 1, 1024, 768, 8, 2
+    q, k, v, dout, scale = _inputs(B, Sq, Skv, Hq, Hkv, seed=3)
+    qd, kd, vd, dod = (t.to(gpu) for t in (q, k, v, dout))
+    o, lse = _mla_fwd(qd, kd, vd, scale, False)
+    delta = _mla_bwd_preprocess(o, dod)
+    monkeypatch.setattr(H, "ds_plan", lambda *a: (Hkv, attn_bwd_ds_bytes(qd, kd, vd, False)))
+    need = attn_bwd_ds_bytes(qd, kd, vd, False)
+    real_empty = torch.empty
+
+    def failing_empty(*a, **kw):  # only the hand-over buffer's allocation fails
+        if a and a[0] == need and kw.get("dtype") == torch.uint8:
+            raise torch.cuda.OutOfMemoryError("forced by the test")
+        return real_empty(*a, **kw)
+
+    out = {}
+    for name in ("handover", "oom"):
+        with monkeypatch.context() as m:
+            if name == "oom":
+                m.setattr(torch, "empty", failing_empty)
+            dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+            used = H.attn_bwd_pair_into(qd, kd, vd, dod, lse, delta, dq, dk, dv, scale, False)
+        out[name] = (dq, dk, dv, used)
+    assert out["handover"][3] > 0 and out["oom"][3] == 0
+    assert torch.equal(out["handover"][1], out["oom"][1]) and torch.equal(out["handover"][2], out["oom"][2])
+    rdq, _, _ = R.chunk_bwd(q, k, v, dout, lse.double().cpu(), delta.double().cpu(), scale, False)
+    check_bf16_result(out["oom"][0], rdq, "recomputed dQ after allocation failure", otol=1e-3)
+    check_bf16_result(out["handover"][0], rdq, "hand-over dQ", otol=1e-3)

@@ -163,3 +163,40 @@ def test_reference_entry_points_with_a_process_group(gpu, one_rank_group):
         check_bf16_result(qd.grad, dq_ref, "dQ", otol=1e-3)
         check_bf16_result(kd.grad, dk_ref, "dK", otol=1e-3)
         check_bf16_result(vd.grad, dv_ref, "dV", otol=1e-3)
+
+
+def test_autograd_functions_with_the_references_seven_arguments(gpu):
+    """RingAttentionFunc.apply / RingMLAAttentionFunc.apply called with exactly the reference's seven positional
+    arguments (q, k, v, softmax_scale, cp_rank, cp_size, global_ranks: standard.py:73, mla.py:47); the backward
+    returns seven gradients (standard.py:189, mla.py:149): dq, dk, dv and four None."""
+    from pithtrain_amd.operators.ring_attention.mla import RingMLAAttentionFunc
+    from pithtrain_amd.operators.ring_attention.standard import RingAttentionFunc
+
+    for base, (H, Hkv, DQ, DV) in ((RingAttentionFunc, (8, 2, 128, 128)), (RingMLAAttentionFunc, (4, 4, 192, 128))):
+        returned = []
+
+        class Probe(base):
+            @staticmethod
+            def backward(ctx, dout):
+                grads = base.backward(ctx, dout)
+                returned.append(grads)
+                return grads
+
+        B, S = 2, 320
+        torch.manual_seed(5)
+        q = torch.randn(B, S, H, DQ, dtype=torch.bfloat16)
+        k = torch.randn(B, S, Hkv, DQ, dtype=torch.bfloat16)
+        v = torch.randn(B, S, Hkv, DV, dtype=torch.bfloat16)
+        dout = torch.randn(B, S, H, DV, dtype=torch.bfloat16)
+        scale = DQ**-0.5
+        qd, kd, vd = (t.to(gpu).requires_grad_(True) for t in (q, k, v))
+        out = Probe.apply(qd, kd, vd, scale, 0, 1, [0])
+        assert out.dtype == torch.bfloat16 and tuple(out.shape) == (B, S, H, DV)
+        out.backward(dout.to(gpu))
+        (grads,) = returned
+        assert len(grads) == 7 and all(g is None for g in grads[3:]), "backward must return the reference's 7-tuple"
+        o_ref, lse_ref, dq_ref, dk_ref, dv_ref = _full_reference(q, k, v, dout, scale)
+        check_bf16_result(out, o_ref, "O")
+        check_bf16_result(qd.grad, dq_ref, "dQ", otol=1e-3)
+        check_bf16_result(kd.grad, dk_ref, "dK", otol=1e-3)
+        check_bf16_result(vd.grad, dv_ref, "dV", otol=1e-3)

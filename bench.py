@@ -2,22 +2,27 @@
 """Benchmark of the ring-attention hot path on ONE MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra-configs]
-    python bench.py --config mla16k|long131k [--steps K]     (one of the other configurations alone)
+    python bench.py --config mla16k|long131k|mla_op [--steps K]     (one of the other configurations alone)
 
 A step is one forward + backward pass of one GPU's share of causal ring attention at the
 Qwen3-30B-A3B shape (32 q heads / 4 kv heads, head dim 128, 32768 tokens as 4 zigzag chunks of 8192,
 rank 1 of 4): 4 chunk-attention forwards, 3 log2 combines, delta, 4 dK/dV and 4 dQ launches.
 Inputs are synthetic (CPU generator, seed 42; q/k/v ~ N(0,1)/sqrt(Dqk), dO ~ N(0,1)) and resident in
-HBM before the timed region. One JSON line is printed; everything in it is measured in this run
-except the block under "from_profiles", which quotes hardware-counter figures of earlier rocprofv3
-runs by file:
+HBM before the timed region. One JSON line is printed; everything in it is measured in this run except
+`roofline.traffic` (HBM bytes per launch need a rocprofv3 --pmc run: the figure is read from the committed summary
+named beside it in `traffic_from`, null when that summary has none):
 
   value      algorithmic TFLOP/s of the whole step: 2*(Dqk+Dv)*E*Hq forward + 2*(3Dqk+2Dv)*E*Hq backward
              with E = C*S_l^2/2 score entries per head (5 backward matmuls; recomputation not counted)
-  fwd_only   the forward alone (the forward-only configuration of the same shape)
   roofline   the dominant kernel (non-causal dK/dV), timed per launch with events on the launch stream
-  mla16k     the same ring driver at the MLA shape (16 heads, 192/128, 16384 tokens as 4 zigzag chunks)
-  long131k   the same at the long-context shape (64 q / 4 kv heads, 131072 tokens as 8 zigzag chunks, rank 3)
+  fwd_only   the forward alone (the forward-only configuration of the same shape), with its dominant kernel
+             (the non-causal forward launch) and its own CPU baseline
+  mla16k     the same ring driver at the MLA shape (16 heads, 192/128, 16384 tokens as 4 zigzag chunks), with the
+             roofline of its dominant kernel and the CPU port on the whole workload
+  long131k   the same at the long-context shape (64 q / 4 kv heads, 131072 tokens as 8 zigzag chunks, rank 3);
+             CPU port on 4 of the 64 query heads
+  mla_op     the reference's own MLA operator benchmark matrix (h in {16,128} x s in {4096,32768}, causal,
+             forward and backward) with its FLOP and byte models
   combine    the log2 combine at [1,4096,32,128] bf16+bf16 -> fp32 over rotating buffers, GB/s of
              algorithmic bytes against the 8 TB/s HBM peak: timed as replays of a captured HIP graph
              (kernel time, no host launch cost in between) and, beside it, launched eagerly
@@ -44,27 +49,25 @@ HBM_PEAK_GBPS = 8000.0
 
 HQ, HKV, DQK, DV, S_LOCAL, CP, RANK = 32, 4, 128, 128, 8192, 4, 1
 LAYOUT = "zigzag"
-COMBINE_TRAFFIC = 135_900_000
 
 
-# Figures that are NOT measured by this program: hardware-counter results of rocprofv3 --pmc runs over
-# `bench.py --counter-pass`, kept here only so that the JSON line can point at them. They describe the
-# kernels as they were when the named summary was written.
-FROM_PROFILES = {
-    "note": "quoted from committed rocprofv3 summaries, not measured in this run",
-    "attn_bwd_dkdv_d128_kernel<non-causal>": {
-        "file": "profiles/attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt",
-        # with the dS stores: 153.4 MB fetched + 2169.9 MB written (2147.5 MB of dS, the rest dK / dV or their head-split partials)
-        "hbm_bytes_per_launch": 2_323_000_000,
-        "hbm_bytes_per_launch_without_ds_stores": 175_700_000,  # 153.4 MB fetched + 22.4 MB written (mean of the three launches)
-        "mfma_file": "profiles/attn_kernels_mfma_lds_counters.txt",
-        "mfma_busy_fraction": 0.58,  # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs); 0.68 without the stores
-        "sustained_clock_ghz": 1.75,  # GRBM_GUI_ACTIVE / 8 XCDs / launch duration (2.4 GHz nominal); 1.85 without the stores
-    },
-    "combine_front_kernel": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_per_launch": COMBINE_TRAFFIC},
-    "norm_rope_kernels": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_fwd_plus_bwd": 159_400_000 + 235_200_000},
-    "mla_assemble_kernels": {"file": "profiles/combine_norm_rope_mla_assemble_hbm_counters.txt", "hbm_bytes_fwd_plus_bwd": 128_000_000 + 128_000_000},
-}
+def profile_figure(name, key):
+    """A figure quoted from a committed rocprofv3 summary: the value of the line `bench.py <key> = <number>` in
+    profiles/<name>, or None when the file or the line is missing. HBM traffic cannot be measured by this
+    program (it needs a rocprofv3 --pmc run), so `roofline.traffic` is read from the summary of that run."""
+    try:
+        with open(os.path.join(ROOT, "profiles", name)) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) >= 4 and parts[0] == "bench.py" and parts[1] == key and parts[2] == "=":
+                    return int(float(parts[3]))
+    except OSError:
+        pass
+    return None
+
+
+HBM_COUNTERS = "attn_bwd_dkdv_d128_qwen3_step_hbm_counters.txt"
+STREAM_COUNTERS = "combine_norm_rope_mla_assemble_hbm_counters.txt"
 
 
 class RingConfig:
@@ -188,57 +191,160 @@ def handover_scratch_bytes(cfg, dev):
     return most
 
 
-def bench_other_config(torch, device, cfg, steps, warmup):
-    _, dev = cfg.make_inputs(torch, device)
-    ms_step, ms_fwd, ms_bwd, _, _ = time_ring_share(torch, cfg, dev, steps, warmup)
-    out = ring_summary(cfg, ms_step, ms_fwd, ms_bwd)
-    out["ds_handover_scratch_bytes_per_ring_step"] = handover_scratch_bytes(cfg, dev)
-    del dev
-    torch.cuda.empty_cache()
+def roofline_entry(kernel, flops_per_launch, ms_per_launch, launches, traffic=None, traffic_from=None, note=None):
+    tf = flops_per_launch / (ms_per_launch * 1e-3) / 1e12
+    out = {
+        "kernel": kernel, "bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic, "traffic_from": traffic_from,
+        "ms_per_launch": round(ms_per_launch, 4), "flop_per_launch": flops_per_launch, "launches_per_step": launches,
+    }  # fmt: skip
+    if note:
+        out["note"] = note
     return out
 
 
-def bench_ring(torch, args, dev_inputs):
-    from pithtrain_amd.operators.mla.hip import attn_bwd_delta_into, attn_bwd_dkdv_into, ds_buffer
+def noncausal_steps(cfg):
     from pithtrain_amd.operators.ring_attention.local import ring_schedule
 
-    q, ks, vs, dout = dev_inputs
-    scale = DQK**-0.5
-    ms_step, ms_fwd, ms_bwd, out, lse = time_ring_share(torch, QWEN3, dev_inputs, args.steps, args.warmup)
+    return [s for s in ring_schedule(cfg.rank, cfg.cp, cfg.s_local, LAYOUT) if not s.causal]
 
-    # Dominant kernel: the non-causal dK/dV launch (3 per step; every one covers S_l^2/2 score
-    # entries per query head and performs 4 of the 5 algorithmic backward products).
+
+def dominant_dkdv(torch, cfg, dev, out, lse, reps, counter_pass=False):
+    """The non-causal dK/dV launches of one step of `cfg`, launched exactly as the ring backward launches them
+    (with the dS hand-over buffer, whole or one slab of kv heads at a time, whenever its policy takes one) and
+    timed with events on the launch stream. Returns (ms per launch, FLOP per launch, launches per step, bytes of
+    hand-over scratch)."""
+    from pithtrain_amd.operators.mla import hip
+
+    q, ks, vs, dout = dev
+    scale = cfg.dqk**-0.5
     delta = torch.empty_like(lse)
-    attn_bwd_delta_into(out, dout, delta)
-    st = [s for s in ring_schedule(RANK, CP, S_LOCAL, LAYOUT) if not s.causal]
-    launches = []
-    for s in st:
-        k_j, v_j = ks[s.kv_rank][:, s.kv_rows[0] : s.kv_rows[1]], vs[s.kv_rank][:, s.kv_rows[0] : s.kv_rows[1]]
-        rows = slice(s.q_rows[0], s.q_rows[1])
+    hip.attn_bwd_delta_into(out, dout, delta)
+    launches, buf, flops = [], None, 0
+    for s in noncausal_steps(cfg):
+        kr, qr = slice(*s.kv_rows), slice(*s.q_rows)
+        k_j, v_j = ks[s.kv_rank][:, kr], vs[s.kv_rank][:, kr]
         dk, dv = torch.empty_like(k_j), torch.empty_like(v_j)
-        launches.append((q[:, rows], k_j, v_j, dout[:, rows], lse[:, :, rows], delta[:, :, rows], dk, dv))
-    # the same kernel variant as in the step: with the dS hand-over buffer whenever the ring driver would use one
-    hand = ds_buffer(*launches[0][:3])
+        plan = hip.ds_plan(q[:, qr], k_j, v_j, False)
+        if plan is not None and buf is None:
+            buf = hip._try_alloc(plan[1], q.device)
+        heads = plan[0] if plan is not None and buf is not None else cfg.hkv
+        g = cfg.hq // cfg.hkv
+        for h0 in range(0, cfg.hkv, heads):
+            kv_h, q_h = slice(h0, h0 + heads), slice(h0 * g, (h0 + heads) * g)
+            launches.append((q[:, qr, q_h], k_j[:, :, kv_h], v_j[:, :, kv_h], dout[:, qr, q_h], lse[:, q_h, qr],
+                             delta[:, q_h, qr], dk[:, :, kv_h], dv[:, :, kv_h]))  # fmt: skip
+        flops = 2 * (2 * cfg.dqk + 2 * cfg.dv) * (qr.stop - qr.start) * (kr.stop - kr.start) * heads * g
 
-    def dkdv_launches():
+    def run():
         for a in launches:
-            attn_bwd_dkdv_into(*a, scale, False, ds=hand)
+            hip.attn_bwd_dkdv_into(*a, scale, False, ds=buf)
 
-    dkdv_launches()
-    if args.counter_pass:
-        # rocprofv3 --pmc run: a few more launches of the roofline kernel and a plain elementwise
-        # copy of known size (256 MiB read, 256 MiB written) to calibrate the counter against
-        dkdv_launches()
-        src = torch.ones(64 << 20, dtype=torch.float32, device=q.device)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            torch.mul(src, 1.0, out=dst)
+    run()
+    if counter_pass:
+        run()
         torch.cuda.synchronize()
         return None
-    ms_dkdv = time_events(torch, dkdv_launches, args.steps) / len(launches)
-    entries = (S_LOCAL * S_LOCAL // 2) * HQ
-    dkdv_flops = 2 * (2 * DQK + 2 * DV) * entries
-    return ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops, hand is not None
+    ms = time_events(torch, run, reps) / len(launches)
+    return ms, flops, len(launches), (0 if buf is None else buf.numel())
+
+
+def dominant_fwd(torch, cfg, dev, reps):
+    """The non-causal chunk-attention forward launches of one step of `cfg`, timed like dominant_dkdv."""
+    from pithtrain_amd.operators.mla import hip
+
+    q, ks, vs, _ = dev
+    scale = cfg.dqk**-0.5
+    launches, flops = [], 0
+    for s in noncausal_steps(cfg):
+        kr, qr = slice(*s.kv_rows), slice(*s.q_rows)
+        n_q = qr.stop - qr.start
+        o = torch.empty((1, n_q, cfg.hq, cfg.dv), dtype=torch.bfloat16, device=q.device)
+        l = torch.empty((1, cfg.hq, n_q), dtype=torch.float32, device=q.device)
+        launches.append((q[:, qr], ks[s.kv_rank][:, kr], vs[s.kv_rank][:, kr], o, l))
+        flops = 2 * (cfg.dqk + cfg.dv) * n_q * (kr.stop - kr.start) * cfg.hq
+
+    def run():
+        for a in launches:
+            hip.attn_fwd_into(*a, scale, False)
+
+    run()
+    return time_events(torch, run, reps) / len(launches), flops, len(launches)
+
+
+def bench_other_config(torch, device, cfg, steps, warmup, cpu_heads=None, counter_pass=False):
+    """Step time of another configuration through the same ring driver, its dominant kernel (the non-causal dK/dV
+    launch) against the MFMA roofline, and (cpu_heads = (first, last+1) query heads, or "all") the oracle's CPU port
+    on that sample of the same workload."""
+    host, dev = cfg.make_inputs(torch, device, host=cpu_heads is not None)
+    ms_step, ms_fwd, ms_bwd, o, lse = time_ring_share(torch, cfg, dev, steps, warmup)
+    if counter_pass:
+        dominant_dkdv(torch, cfg, dev, o, lse, 1, counter_pass=True)
+        return None
+    out = ring_summary(cfg, ms_step, ms_fwd, ms_bwd)
+    ms, flops, n, scratch = dominant_dkdv(torch, cfg, dev, o, lse, steps)
+    kname = "attn_bwd_dkdv_d192_kernel" if cfg.dqk == 192 else "attn_bwd_dkdv_d128_kernel"
+    slabs = n // len(noncausal_steps(cfg))
+    out["roofline"] = roofline_entry(
+        f"{kname}<non-causal> (S, dP, dV, dK of one ring step" + (f", one of {slabs} kv-head slabs per launch" if slabs > 1 else "")
+        + ("; also stores its dS tiles for the dQ kernel)" if scratch else ")"),
+        flops, ms, n, profile_figure(HBM_COUNTERS, f"{cfg.name}.dkdv_traffic_bytes_per_launch"), "profiles/" + HBM_COUNTERS)  # fmt: skip
+    out["ds_handover_scratch_bytes_per_ring_step"] = handover_scratch_bytes(cfg, dev)
+    del dev, o, lse
+    torch.cuda.empty_cache()
+    if cpu_heads is not None:
+        out["cpu_baseline"] = cpu_baseline_ring(torch, cfg, host, None if cpu_heads == "all" else cpu_heads)
+    return out
+
+
+def bench_mla_op(torch, device, reps=5):
+    """The reference's own operator benchmark matrix (benchmarks/operators/mla/test_triton.py:41-48): the causal
+    MLA operator, b=1, h in {16, 128}, s in {4096, 32768}, head dims 192/128, forward and backward, with its FLOP
+    and byte models (:7-28, :77-78, :116-118): forward b*h*s^2*(dq+dv), backward 2.5x that."""
+    from pithtrain_amd.operators.mla.hip import MLA
+
+    dq, dv = 192, 128
+    rows = []
+    for h in (16, 128):
+        for s in (4096, 32768):
+            torch.manual_seed(42)
+            q = torch.randn((1, s, h, dq), dtype=torch.bfloat16, device=device, requires_grad=True)
+            k = torch.randn((1, s, h, dq), dtype=torch.bfloat16, device=device, requires_grad=True)
+            v = torch.randn((1, s, h, dv), dtype=torch.bfloat16, device=device, requires_grad=True)
+            do = torch.randn((1, s, h, dv), dtype=torch.bfloat16, device=device)
+            op = MLA(h, dq, dv, dq**-0.5)
+
+            def fwd():
+                with torch.no_grad():
+                    return op.forward(q, k, v)
+
+            o = op.forward(q, k, v)
+
+            def bwd():
+                q.grad = k.grad = v.grad = None
+                o.backward(do, retain_graph=True)
+
+            fwd(), bwd()
+            n = reps if s > 4096 else 4 * reps
+            ms_f, ms_b = time_events(torch, fwd, n), time_events(torch, bwd, n)
+            f_flops = h * s * s * (dq + dv)
+            b_flops = int(2.5 * f_flops)
+            f_bytes = s * h * (dq * 4 + dv * 4) + h * s * 4
+            b_bytes = s * h * (dq * 8 + dv * 6) + h * s * 8
+            rows.append({
+                "b": 1, "s": s, "h": h, "dq": dq, "dv": dv,
+                "fwd": {"ms": round(ms_f, 4), "tflops": round(f_flops / ms_f / 1e9, 1), "tbps": round(f_bytes / ms_f / 1e9, 3),
+                        "frac_mfma_peak": round(f_flops / ms_f / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)},
+                "bwd": {"ms": round(ms_b, 4), "tflops": round(b_flops / ms_b / 1e9, 1), "tbps": round(b_bytes / ms_b / 1e9, 3),
+                        "frac_mfma_peak": round(b_flops / ms_b / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)},
+            })  # fmt: skip
+            del q, k, v, do, o
+            torch.cuda.empty_cache()
+    return {
+        "what": "causal MLA operator (module MLA, autograd backward = delta + dK/dV + dQ), the reference's benchmark "
+                "matrix and FLOP / byte models (benchmarks/operators/mla/test_triton.py)",
+        "rows": rows,
+    }  # fmt: skip
 
 
 def bench_combine(torch, device, reps=50, graph=True):
@@ -394,16 +500,27 @@ def cpu_baseline_norm_rope(torch, host, reps=3):
     return nbytes / times[len(times) // 2] / 1e9
 
 
-def cpu_baseline_ring(torch, host_inputs):
-    """The whole configuration once on the host cores: every head, every row."""
+def cpu_baseline_ring(torch, cfg, host_inputs, heads=None, backward=True):
+    """The oracle's blocked fp32 eager-PyTorch port of the same ring share on the host cores, once: all query
+    heads, or the sample heads = (first, last + 1) (whole kv-head groups), whose work is a fixed fraction of the
+    configuration's (every head does the same work) and is counted as such."""
     from oracle import ring_oracle as R
 
     q, ks, vs, dout = host_inputs
+    h0, h1 = heads if heads is not None else (0, cfg.hq)
     t0 = time.perf_counter()
-    R.cpu_ring_fwd_bwd(q, ks, vs, dout, DQK**-0.5, RANK, CP, LAYOUT, heads=(0, HQ), q_block=1024)
+    R.cpu_ring_fwd_bwd(q, ks, vs, dout, cfg.dqk**-0.5, cfg.rank, cfg.cp, LAYOUT, heads=(h0, h1), q_block=1024, backward=backward)
     dt = time.perf_counter() - t0
-    fwd, bwd = flops_per_step()
-    return (fwd + bwd) / dt / 1e12, dt
+    fwd, bwd = cfg.flops()
+    work = (fwd + (bwd if backward else 0)) * (h1 - h0) / cfg.hq
+    what = "forward + backward" if backward else "forward only"
+    sample = (f"the whole workload once (all {cfg.hq} query heads, all rows, {what})" if (h0, h1) == (0, cfg.hq) else
+              f"query heads {h0}..{h1 - 1} of {cfg.hq} (of kv head {h0 // (cfg.hq // cfg.hkv)}), all rows, {what}: "
+              f"{h1 - h0}/{cfg.hq} of the workload's FLOP, counted as such (the whole is not extrapolated from it)")  # fmt: skip
+    return {
+        "value": round(work / dt / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"{sample}, fp32 eager PyTorch on bf16-rounded inputs, {dt:.1f} s; os.cpu_count()={os.cpu_count()}",
+    }  # fmt: skip
 
 
 def cpu_baseline_combine(torch, host, nbytes, reps=5):
@@ -426,8 +543,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-configs", action="store_true",
                     help="skip the MLA 16K and long 131K configurations (sub-objects mla16k, long131k)")
-    ap.add_argument("--config", choices=["mla16k", "long131k"], default=None,
-                    help="time only this configuration's ring share and print its sub-object (for kernel traces)")
+    ap.add_argument("--config", choices=["mla16k", "long131k", "mla_op"], default=None,
+                    help="time only this configuration (ring share, or the MLA operator matrix) and print its sub-object "
+                         "(for kernel traces)")
     ap.add_argument("--no-handover", action="store_true",
                     help="run everything with the dS hand-over between the backward kernels switched off (for traces)")
     ap.add_argument("--counter-pass", action="store_true",
@@ -449,34 +567,51 @@ def main():
         from pithtrain_amd.operators.mla import hip
 
         hip.DS_BUFFER_LIMIT_BYTES = 0
+    cpu_on = not args.no_cpu_baseline
     if args.config:
+        if args.config == "mla_op":
+            print(json.dumps({"mla_op": bench_mla_op(torch, device)}))
+            return
         cfg = MLA16K if args.config == "mla16k" else LONG131K
-        print(json.dumps({args.config: bench_other_config(torch, device, cfg, args.steps, args.warmup)}))
+        res = bench_other_config(torch, device, cfg, args.steps, args.warmup, counter_pass=args.counter_pass)
+        print(json.dumps({args.config: res}) if res is not None else "counter pass done")
         return
     host_inputs, dev_inputs = make_inputs(torch, device)
-    ring = bench_ring(torch, args, dev_inputs)
-    if ring is None:
-        # the HBM-bound kernels, a few dispatches each, for the same counters
-        del dev_inputs
-        bench_other_config(torch, device, MLA16K, 1, 0)  # the 192/128 kernels, for the same counters
+    ms_step, ms_fwd, ms_bwd, out, lse = time_ring_share(torch, QWEN3, dev_inputs, args.steps, args.warmup)
+    if args.counter_pass:
+        # rocprofv3 --pmc run: a few more launches of the roofline kernel, a plain elementwise copy of known size
+        # (256 MiB read, 256 MiB written) to calibrate the counter against, and the other kernels a few times each
+        dominant_dkdv(torch, QWEN3, dev_inputs, out, lse, 1, counter_pass=True)
+        src = torch.ones(64 << 20, dtype=torch.float32, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del dev_inputs, out, lse, src, dst
+        bench_other_config(torch, device, MLA16K, 1, 0, counter_pass=True)
         bench_combine(torch, device, reps=4, graph=False)
         bench_norm_rope(torch, device, reps=3)
         bench_mla_assemble(torch, device, reps=3)
         print("counter pass done")
         return
-    ms_step, ms_fwd, ms_bwd, ms_dkdv, dkdv_flops, handover_on = ring
+    ms_dkdv, dkdv_flops, dkdv_n, scratch = dominant_dkdv(torch, QWEN3, dev_inputs, out, lse, args.steps)
+    ms_fwdk, fwdk_flops, fwdk_n = dominant_fwd(torch, QWEN3, dev_inputs, args.steps)
+    handover_on = scratch > 0
+    scratch = handover_scratch_bytes(QWEN3, dev_inputs)
     recompute = None
     if not args.no_extra_configs and handover_on:
         recompute = bench_recompute(torch, dev_inputs, args.steps, args.warmup)
-    scratch = handover_scratch_bytes(QWEN3, dev_inputs) if handover_on else 0
-    del dev_inputs
+    del dev_inputs, out, lse
     torch.cuda.empty_cache()
     fwd_flops, bwd_flops = flops_per_step()
     tflops = (fwd_flops + bwd_flops) / (ms_step * 1e-3) / 1e12
-    mla16k = long131k = None
+    mla16k = long131k = mla_op = None
     if not args.no_extra_configs:
-        mla16k = bench_other_config(torch, device, MLA16K, args.steps, args.warmup)
-        long131k = bench_other_config(torch, device, LONG131K, max(2, args.steps // 5), 1)
+        mla16k = bench_other_config(torch, device, MLA16K, args.steps, args.warmup, cpu_heads="all" if cpu_on else None)
+        # CPU sample of the long configuration: 4 of its 64 query heads (a quarter of one kv-head group; a whole
+        # group would be ~90 s of host time)
+        long131k = bench_other_config(torch, device, LONG131K, max(2, args.steps // 5), 1, cpu_heads=(0, 4) if cpu_on else None)
+        mla_op = bench_mla_op(torch, device)
     ms_comb, ms_comb_eager, comb_bytes, comb_host = bench_combine(torch, device)
     comb_gbps = comb_bytes / (ms_comb * 1e-3) / 1e9
     nr_ms_f, nr_bytes_f, nr_ms_b, nr_bytes_b, nr_host = bench_norm_rope(torch, device)
@@ -485,16 +620,10 @@ def main():
     ma_gbps = (ma_bytes_f + ma_bytes_b) / ((ma_ms_f + ma_ms_b) * 1e-3) / 1e9
 
     cores = torch.get_num_threads()
-    cpu = None
-    combine_cpu = None
-    norm_rope_cpu = None
-    if not args.no_cpu_baseline:
-        cpu_tflops, cpu_s = cpu_baseline_ring(torch, host_inputs)
-        cpu = {
-            "value": round(cpu_tflops, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"the whole workload once (all {HQ} query heads, all rows, forward + backward), fp32 eager PyTorch "
-                      f"on bf16-rounded inputs, {cpu_s:.1f} s; os.cpu_count()={os.cpu_count()}",
-        }  # fmt: skip
+    cpu = fwd_cpu = combine_cpu = norm_rope_cpu = None
+    if cpu_on:
+        cpu = cpu_baseline_ring(torch, QWEN3, host_inputs)
+        fwd_cpu = cpu_baseline_ring(torch, QWEN3, host_inputs, backward=False)
         combine_cpu = {
             "value": round(cpu_baseline_combine(torch, comb_host, comb_bytes), 2), "unit": "GB/s", "cores": cores,
             "kind": "port", "sample": "full [1,4096,32,128] combine, eager PyTorch, median of 5",
@@ -504,8 +633,6 @@ def main():
             "sample": "q tensor [1,8192,32,128] only, forward + backward, fp32 eager PyTorch, median of 3",
         }  # fmt: skip
 
-    dkdv_tflops = dkdv_flops / (ms_dkdv * 1e-3) / 1e12
-    dkdv_prof = FROM_PROFILES["attn_bwd_dkdv_d128_kernel<non-causal>"]
     line = {
         "metric": "ring-attn fwd+bwd causal TFLOP/s (Qwen3-30B-A3B, 32K)",
         "value": round(tflops, 2),
@@ -528,19 +655,19 @@ def main():
         "fwd": {"ms": round(ms_fwd, 4), "tflops": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2)},
         "bwd": {"ms": round(ms_bwd, 4), "tflops": round(bwd_flops / (ms_bwd * 1e-3) / 1e12, 2)},
         "fwd_only": {
-            "workload": "the same share, forward only (4 chunk-attention launches + 3 combines): O and the base-2 LSE",
+            "workload": "the same share, forward only (4 chunk-attention launches and the log2 merges): O and the base-2 LSE",
             "ms": round(ms_fwd, 4), "tflops": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2),
             "frac_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-        },
-        "roofline": {
-            "kernel": "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step"
-                      + ("; also stores its dS tiles for the dQ kernel)" if handover_on else ")"),
-            "bound": "mfma", "achieved": round(dkdv_tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": dkdv_prof["hbm_bytes_per_launch" if handover_on else "hbm_bytes_per_launch_without_ds_stores"],
-            "traffic_from": dkdv_prof["file"],
-            "ms_per_launch": round(ms_dkdv, 4),
+            "roofline": roofline_entry(
+                "attn_fwd_direct_kernel<128, non-causal> (S, P, O of one ring step)", fwdk_flops, ms_fwdk, fwdk_n,
+                profile_figure(HBM_COUNTERS, "qwen3-32k.fwd_traffic_bytes_per_launch"), "profiles/" + HBM_COUNTERS),
+            "cpu_baseline": fwd_cpu,
         },  # fmt: skip
+        "roofline": roofline_entry(
+            "attn_bwd_dkdv_d128_kernel<non-causal> (S, dP, dV, dK of one ring step"
+            + ("; also stores its dS tiles for the dQ kernel)" if handover_on else ")"), dkdv_flops, ms_dkdv, dkdv_n,
+            profile_figure(HBM_COUNTERS, "qwen3-32k.dkdv_traffic_bytes_per_launch" if handover_on
+                           else "qwen3-32k.dkdv_traffic_bytes_per_launch_without_ds_stores"), "profiles/" + HBM_COUNTERS),  # fmt: skip
         "ds_handover": {
             "on": handover_on,
             "what": "the dK/dV kernel hands its dS tiles to the dQ kernel (5 matrix products executed instead of 7)",
@@ -549,6 +676,7 @@ def main():
         },
         "mla16k": mla16k,
         "long131k": long131k,
+        "mla_op": mla_op,
         "combine": {
             "metric": "online_softmax_combine_log2 GB/s ([1,4096,32,128] bf16 x2 -> fp32)",
             "value": round(comb_gbps, 1), "unit": "GB/s", "us_per_launch": round(ms_comb * 1e3, 2),
@@ -558,8 +686,8 @@ def main():
             "bytes": comb_bytes,
             "roofline": {"bound": "hbm", "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": round(comb_gbps / HBM_PEAK_GBPS, 4),
-                         "traffic": FROM_PROFILES["combine_front_kernel"]["hbm_bytes_per_launch"],
-                         "traffic_from": FROM_PROFILES["combine_front_kernel"]["file"]},
+                         "traffic": profile_figure(STREAM_COUNTERS, "combine.traffic_bytes_per_launch"),
+                         "traffic_from": "profiles/" + STREAM_COUNTERS},
             "cpu_baseline": combine_cpu,
         },  # fmt: skip
         "norm_rope": {
@@ -583,7 +711,6 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(ma_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": round(ma_gbps / HBM_PEAK_GBPS, 4)},
         },  # fmt: skip
-        "from_profiles": FROM_PROFILES,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

@@ -227,19 +227,22 @@ def ring_backward(dout, q, combined_out, combined_lse, k_chunks: Sequence, v_chu
 
 
 def cpu_ring_fwd_bwd(q, k_chunks, v_chunks, dout, scale, cp_rank, cp_size, layout,
-                     heads: Optional[Tuple[int, int]] = None, q_block: int = 1024):  # fmt: skip
+                     heads: Optional[Tuple[int, int]] = None, q_block: int = 1024, backward: bool = True):  # fmt: skip
     """Forward + backward of one rank in fp32 on bf16-rounded inputs, for query heads
     [heads[0], heads[1]) only (all when None). Score tiles are [heads, q_block, Skv] at most.
     Returns (out, lse, dq, dk_list, dv_list) restricted to those heads (kv gradients hold only the
-    contribution of those query heads)."""
+    contribution of those query heads). backward=False stops after the forward (the gradients
+    returned are then meaningless)."""
     hq, hkv = q.shape[2], k_chunks[cp_rank].shape[2]
     g = hq // hkv
     h0, h1 = heads if heads is not None else (0, hq)
-    assert h0 % g == 0 and h1 % g == 0, "head range must cover whole kv groups"
+    whole_groups = h0 % g == 0 and h1 % g == 0
+    assert whole_groups or h0 // g == (h1 - 1) // g, "head range must cover whole kv groups or lie within one"
+    kv0, kv1 = h0 // g, (h1 - 1) // g + 1
     f32 = torch.float32
     qh, doh = q[:, :, h0:h1].to(f32), dout[:, :, h0:h1].to(f32)
-    ks = [None if c is None else c[:, :, h0 // g : h1 // g].to(f32) for c in k_chunks]
-    vs = [None if c is None else c[:, :, h0 // g : h1 // g].to(f32) for c in v_chunks]
+    ks = [None if c is None else c[:, :, kv0:kv1].to(f32) for c in k_chunks]
+    vs = [None if c is None else c[:, :, kv0:kv1].to(f32) for c in v_chunks]
     S = q.shape[1]
     out = torch.empty((q.shape[0], S, h1 - h0, vs[cp_rank].shape[-1]), dtype=f32)
     lse = torch.empty((q.shape[0], h1 - h0, S), dtype=f32)
@@ -259,6 +262,8 @@ def cpu_ring_fwd_bwd(q, k_chunks, v_chunks, dout, scale, cp_rank, cp_size, layou
             no, nl = combine_log2(co[:, a - r0 : b - r0], cl[:, :, a - r0 : b - r0], so, sl)
             co[:, a - r0 : b - r0], cl[:, :, a - r0 : b - r0] = no, nl
         out[:, r0:r1], lse[:, :, r0:r1] = co, cl
+        if not backward:
+            continue
         delta = bwd_delta(co.to(torch.bfloat16), doh[:, r0:r1], f32)
         dq[:, r0:r1] = 0
         for j, causal, (a, b), (n0, n1) in sub:

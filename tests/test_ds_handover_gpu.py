@@ -176,21 +176,29 @@ def test_default_policy_of_the_buffer(gpu, monkeypatch):
     assert buf is not None and buf.numel() == 1 << 30 and buf.data_ptr() % 256 == 0
     del buf
     monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (1 << 30) - 1)
-    assert H.ds_plan(*big) == (2, 1 << 29) and ds_buffer(*big) is None  # two slabs of two kv heads
-    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (1 << 28) + 5)
-    assert H.ds_plan(*big) == (1, 1 << 28)
-    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (1 << 28) - 1)
-    assert H.ds_plan(*big) is None
+    assert H.ds_plan(*big) is None and ds_buffer(*big) is None  # slabs of 2 kv heads: 8 x 16 workgroups, too few
+    # 16384 x 16384 rows, 32 / 4 heads: 4 GiB per kv head, 32 x 8 workgroups of the dQ kernel per kv head
+    q = torch.empty(1, dtype=torch.bfloat16, device=gpu).as_strided((1, 16384, 32, 128), (0, 0, 0, 0))
+    k = torch.empty(1, dtype=torch.bfloat16, device=gpu).as_strided((1, 16384, 4, 128), (0, 0, 0, 0))
+    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", 16 << 30)
+    assert H.ds_plan(q, k, k) == (4, 16 << 30)
+    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (16 << 30) - 1)
+    assert H.ds_plan(q, k, k) == (2, 8 << 30) and ds_buffer(q, k, k) is None  # two slabs of two kv heads
+    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (4 << 30) + 5)
+    assert H.ds_plan(q, k, k) == (1, 4 << 30)
+    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", (4 << 30) - 1)
+    assert H.ds_plan(q, k, k) is None
     # the 131072-token configuration (64 / 4 heads, 16384 x 8192 rows per ring step): one kv head at a time
     monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", 4 << 30)
-    q = torch.empty(1, dtype=torch.bfloat16, device=gpu).as_strided((1, 16384, 64, 128), (0, 0, 0, 0))
-    k = torch.empty(1, dtype=torch.bfloat16, device=gpu).as_strided((1, 8192, 4, 128), (0, 0, 0, 0))
-    assert H.ds_plan(q, k, k) == (1, 4 << 30)
+    q64 = torch.empty(1, dtype=torch.bfloat16, device=gpu).as_strided((1, 16384, 64, 128), (0, 0, 0, 0))
+    k8k = torch.empty(1, dtype=torch.bfloat16, device=gpu).as_strided((1, 8192, 4, 128), (0, 0, 0, 0))
+    assert H.ds_plan(q64, k8k, k8k) == (1, 4 << 30)
     # little free memory: the budget follows it
-    monkeypatch.setattr(H.torch.cuda, "mem_get_info", lambda dev=None: (1 << 29, 1 << 38))
+    monkeypatch.setattr(H, "DS_BUFFER_LIMIT_BYTES", 16 << 30)
+    monkeypatch.setattr(H.torch.cuda, "mem_get_info", lambda dev=None: (8 << 30, 1 << 38))
     monkeypatch.setattr(H.torch.cuda, "memory_reserved", lambda dev=None: 0)
     monkeypatch.setattr(H.torch.cuda, "memory_allocated", lambda dev=None: 0)
-    assert H.ds_plan(*big) == (1, 1 << 28)
+    assert H.ds_plan(q, k, k) == (1, 4 << 30)
 
 
 @pytest.mark.parametrize("causal", [False, True])

@@ -112,7 +112,24 @@ int pith_combine(const pith_combine_args* args, pith_stream_t stream);
  * all heads)], pithtrain/models/deepseek_v2_lite.py:448-454, where the reference materialises it
  * with k_pe broadcast to every head. Here k is then k_nope [B,Skv,Hkv,128] and k_pe [B,Skv,64]
  * (batch stride k_pe_bs, row stride k_pe_rs, elements: it may be a column slice of a wider
- * tensor) is read beside it; results equal those of the assembled key. */
+ * tensor) is read beside it; results equal those of the assembled key.
+ *
+ * Merging with a running result (prev_o != NULL): one ring step in one launch. The chunk's
+ * attention result is combined with the running result of the same query rows the way
+ * _online_softmax_combine_log2(prev_o, lse, o_chunk, lse_chunk) combines them
+ * (ring_attention/mla.py:27-40, called per step at mla.py:64-70 / standard.py:95-101): `lse` holds
+ * the running base-2 LSE on entry and the merged LSE on return; prev_o [B,Sq,Hq,Dv] is bf16 or
+ * fp32 (prev_o_dtype; the reference's running output is fp32 by promotion, mla.py:38); the merged
+ * output is written as bf16 to `o` (may be NULL then) and / or as fp32 to acc_o (may be NULL;
+ * at least one of the two), and either may be the same memory as prev_o when the dtypes agree.
+ * When both are given, o_rows / acc_o_rows ([begin, end) query rows of this call, multiples of 32
+ * or Sq; {0, 0} = all rows) restrict which rows each of them receives: a ring step whose first
+ * rows see their last merge (bf16 result) while the others go on (fp32 running value) then writes
+ * every row once.
+ * Saves the chunk result's round trip through memory and the combine launch. Available for head
+ * dims (128,128) and (192,128) without a causal mask (in a ring the causal step is the first one
+ * and has nothing to merge with); otherwise PITH_ERR_UNSUPPORTED (run pith_attn_fwd, then
+ * pith_combine). */
 typedef struct {
   const void* q;
   const void* k;
@@ -126,6 +143,14 @@ typedef struct {
   int32_t causal;
   const void* k_pe;          /* NULL: k holds all Dqk features */
   int64_t k_pe_bs, k_pe_rs;  /* batch / row strides of k_pe, elements */
+  const void* prev_o;        /* NULL: plain forward (o and lse are only written) */
+  int64_t prev_o_bs;         /* batch stride of prev_o, elements */
+  float* acc_o;              /* merging only: fp32 copy of the merged output, or NULL */
+  int64_t acc_o_bs;
+  int32_t prev_o_dtype;      /* PITH_BF16 | PITH_F32 */
+  int32_t reserved0;         /* keep 0 */
+  int64_t o_rows[2];         /* merging: rows that receive o ({0,0} = all) */
+  int64_t acc_o_rows[2];     /* merging: rows that receive acc_o ({0,0} = all) */
 } pith_attn_fwd_args;
 
 int pith_attn_fwd(const pith_attn_fwd_args* args, pith_stream_t stream);

@@ -259,7 +259,8 @@ using namespace pith;
 
 extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) {
   if (!a) return fail(PITH_ERR_NULL_POINTER, "pith_attn_fwd: args is NULL");
-  if (!a->q || !a->k || !a->v || !a->o || !a->lse) return fail(PITH_ERR_NULL_POINTER, "pith_attn_fwd: NULL tensor pointer");
+  if (!a->q || !a->k || !a->v || !a->lse || (!a->o && !(a->prev_o && a->acc_o)))
+    return fail(PITH_ERR_NULL_POINTER, "pith_attn_fwd: NULL tensor pointer");
   if (a->B <= 0 || a->Sq <= 0 || a->Skv <= 0 || a->Hq <= 0 || a->Hkv <= 0)
     return fail(PITH_ERR_BAD_SHAPE, "pith_attn_fwd: B=%lld Sq=%lld Skv=%lld Hq=%lld Hkv=%lld must all be positive",
                 (long long)a->B, (long long)a->Sq, (long long)a->Skv, (long long)a->Hq, (long long)a->Hkv);
@@ -292,6 +293,29 @@ extern "C" int pith_attn_fwd(const pith_attn_fwd_args* a, pith_stream_t stream) 
                   (long long)a->Dqk, (long long)a->Dv);
     if (!aligned16(a->k_pe) || a->k_pe_bs % 8 || a->k_pe_rs % 8 || a->k_pe_rs < 64)
       return fail(PITH_ERR_MISALIGNED, "pith_attn_fwd: k_pe pointer / strides must keep 16-byte alignment (row stride >= 64)");
+  }
+  p.prev_o = a->prev_o; p.prev_f32 = a->prev_o_dtype == PITH_F32; p.prev_bs = a->prev_o_bs;
+  p.acc_o = a->prev_o ? a->acc_o : nullptr; p.acc_bs = a->acc_o_bs;
+  p.o_r0 = p.o_r1 = p.acc_r0 = p.acc_r1 = 0;
+  if (a->prev_o) {
+    if (a->prev_o_dtype != PITH_BF16 && a->prev_o_dtype != PITH_F32)
+      return fail(PITH_ERR_BAD_DTYPE, "pith_attn_fwd: prev_o_dtype %d is not bf16/fp32", a->prev_o_dtype);
+    if (a->causal || a->Dv != 128 || (a->Dqk != 128 && a->Dqk != 192))
+      return fail(PITH_ERR_UNSUPPORTED, "pith_attn_fwd: merging with a running result needs a non-causal call with head dims "
+                  "(128,128) or (192,128); run pith_attn_fwd and pith_combine instead");
+    if (!aligned16(a->prev_o) || a->prev_o_bs % 8 || (a->acc_o && (!aligned16(a->acc_o) || a->acc_o_bs % 8)))
+      return fail(PITH_ERR_MISALIGNED, "pith_attn_fwd: prev_o / acc_o pointers and batch strides must keep 16-byte alignment");
+    const int64_t* ranges[2] = {a->o_rows, a->acc_o_rows};
+    int* dst[2][2] = {{&p.o_r0, &p.o_r1}, {&p.acc_r0, &p.acc_r1}};
+    for (int i = 0; i < 2; ++i) {
+      int64_t r0 = ranges[i][0], r1 = ranges[i][1];
+      if (r0 == 0 && r1 == 0) r1 = a->Sq;
+      if (r0 < 0 || r1 < r0 || r1 > a->Sq || r0 % 32 || (r1 % 32 && r1 != a->Sq))
+        return fail(PITH_ERR_BAD_SHAPE, "pith_attn_fwd: %s = [%lld, %lld) must lie within the %lld query rows on multiples of 32",
+                    i ? "acc_o_rows" : "o_rows", (long long)ranges[i][0], (long long)ranges[i][1], (long long)a->Sq);
+      *dst[i][0] = (int)r0;
+      *dst[i][1] = (int)r1;
+    }
   }
   hipStream_t st = (hipStream_t)stream;
   begin_launch();

@@ -7,6 +7,7 @@ namespace pith {
 
 constexpr int kFwdBlockN = 64;            // keys per LDS tile
 constexpr float kRescaleThreshold = 8.f;  // log2 units, see attn_fwd.hip
+constexpr float kRescaleLimit = 256.f;    // = 2^kRescaleThreshold: the same bound on a P value, tested on row sums (attn_fwd_direct.hip)
 
 struct FwdParams {
   const __bf16* q;
@@ -22,6 +23,15 @@ struct FwdParams {
   // one vector per position shared by all heads (batch / row strides in elements)
   const __bf16* k_pe;
   int64_t k_pe_bs, k_pe_rs;
+  // merge with the running result of the rows (prev_o != nullptr; non-causal direct-load kernels only): prev_o is
+  // bf16 or fp32 (prev_f32), the merged result goes to o (bf16, may be null then) and / or acc_o (fp32, may be null);
+  // lse holds the running LSE on entry and the merged LSE on return
+  const void* prev_o;
+  int prev_f32;
+  int64_t prev_bs;
+  float* acc_o;
+  int64_t acc_bs;
+  int o_r0, o_r1, acc_r0, acc_r1;  // query rows [r0, r1) that receive o / acc_o when merging (multiples of 32, or Sq)
 };
 
 // Forward for head dims (128, 128) and (192, 128) with tiles loaded global -> LDS directly:

@@ -53,6 +53,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   constexpr int kBM = HALF ? 128 : 256;      // query rows per workgroup
   constexpr int kKTile = kTile + (DQK == 192 ? kExtraTile : 0);
   static_assert(DQK == 128 || DQK == 192, "head dims");
+  constexpr bool kSumTest = !(DQK == 192 && !HALF);  // how the softmax decides to refresh its running maximum
   // the tile rings; the epilogue reuses them to turn the output tile (one area per storing wave)
   constexpr int kRings = kSlots * (kKTile + kTile), kTurn = (HALF ? kWaves / 2 : kWaves) * kRowsViaLdsBytes<DVB>;
   __shared__ __attribute__((aligned(1024))) char smem[kRings > kTurn ? kRings : kTurn];
@@ -129,26 +130,33 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
     for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(src + ks * 16);
   }
 
-  // per-lane read offsets inside a tile
-  // k_off[ks]: straight fragment of this wave's first key block, row c, contraction step ks. Steps
-  // 0..7 lie in the 128-feature tile (the next key block: + 32 rows = + 8192 bytes); steps 8.. in
-  // the extra tile behind it, whose row c holds key c in pieces 0-7 and key c + 32 in pieces 8-15
-  // (the next key block: piece + 8, i.e. the offset with bit 7 flipped).
-  int k_off[KS];
-  int v_off[DVB][2];  // transposing reads of feature block i, lower / upper 8 keys (+ 16 keys: + 4096 bytes)
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    if (ks < 8) k_off[ks] = straight_offset128(c, 2 * ks + g) + kvb0 * 32 * kRowBytes128;
-    else k_off[ks] = kTile + straight_offset128(c, 2 * (ks - 8) + g + 8 * kvb0);
-  }
+  // per-lane read offsets inside a tile. The swizzle is an XOR, so every offset is one base XOR a constant; only the
+  // bases live in registers across the loop (refresh_offsets keeps the compiler from hoisting all derived values
+  // back into registers, where they would push accumulators into scratch memory):
+  //   k_off(ks): straight fragment of this wave's first key block, row c, contraction step ks. Steps 0..7 lie in
+  //     the 128-feature tile (the next key block: + 32 rows = + 8192 bytes); steps 8.. in the extra tile behind it,
+  //     whose row c holds key c in pieces 0-7 and key c + 32 in pieces 8-15 (the next key block: piece + 8, i.e.
+  //     the offset with bit 7 flipped);
+  //   v_off(i, hh): transposing reads of feature block i, lower / upper 8 keys (+ 16 keys: + 4096 bytes).
+  int k_base = straight_offset128(c, g) + kvb0 * 32 * kRowBytes128;
+  int x_base = kTile + straight_offset128(c, g + 8 * kvb0);
+  int v_base[2] = {transposed_offset128(0, 0, 0, lane) + kvb0 * 32 * kRowBytes128,
+                   transposed_offset128(0, 1, 0, lane) + kvb0 * 32 * kRowBytes128};
+  // Only the variants that would spill otherwise pay the extra XOR per read (the 256-row causal kernels); the
+  // others let the compiler keep every derived offset in a register.
+  constexpr bool kDeriveOffsets = !HALF && CAUSAL;
+  auto refresh_offsets = [&]() __attribute__((always_inline)) {
+    if constexpr (kDeriveOffsets) {
+      asm volatile("" : "+v"(k_base), "+v"(v_base[0]), "+v"(v_base[1]));
+      if constexpr (DQK == 192) asm volatile("" : "+v"(x_base));
+    }
+  };
+  auto k_off = [&](int ks) __attribute__((always_inline)) { return ks < 8 ? k_base ^ (ks << 5) : x_base ^ ((ks - 8) << 5); };
+  auto v_off = [&](int i, int hh) __attribute__((always_inline)) { return v_base[hh] ^ (i << 6); };
   auto k_frag = [&](const char* ktile, int ks, int kvb) __attribute__((always_inline)) {
-    const int off = ks < 8 ? k_off[ks] + kvb * 32 * kRowBytes128 : (kvb ? k_off[ks] ^ 128 : k_off[ks]);
+    const int off = ks < 8 ? k_off(ks) + kvb * 32 * kRowBytes128 : (kvb ? k_off(ks) ^ 128 : k_off(ks));
     return *reinterpret_cast<const bf16x8*>(ktile + off);
   };
-#pragma unroll
-  for (int i = 0; i < DVB; ++i)
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) v_off[i][hh] = transposed_offset128(0, hh, 32 * i, lane) + kvb0 * 32 * kRowBytes128;
 
   f32x16 oacc[DVB];
 #pragma unroll
@@ -187,40 +195,82 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
           if (key > limit) s[kvb][v] = -INFINITY;
         }
     }
-    float x = s[0][0];
-#pragma unroll
-    for (int kvb = 0; kvb < KVB; ++kvb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) x = fmaxf(x, s[kvb][v]);
-    const float mx = pair_max(x);
-    const bool refresh = (mx - m_run) * p.kappa > kRescaleThreshold;  // true on the first tile (m = -inf)
-    if (__builtin_amdgcn_ballot_w64(refresh) != 0) {                   // wave-uniform
-      const float m_new = fmaxf(m_run, mx);
-      // a row with no visible key so far keeps m = -inf; exp2 of (-inf - -inf) is avoided
-      const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * p.kappa);
-      m_run = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int i = 0; i < DVB; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
-    }
-    const float mk = (m_run == -INFINITY) ? 0.f : m_run * p.kappa;
+    f32x16 e[KVB];
     float rs = 0.f;
+    if constexpr (kSumTest) {
+      // The running maximum is refreshed lazily, and whether a refresh is due is read off the row sum instead of a
+      // maximum over the tile: every term of the sum is >= 0, so a lane's partial sum within kRescaleLimit means that
+      // none of its P values exceeds kRescaleLimit either. The common tile then costs no maximum at all (24 of the
+      // ~140 vector instructions per tile); a tile that fails the test (the first tile of a row, tiles where the scores
+      // still climb, and any overflow or NaN) is redone from the scores, which are kept until the test has passed.
+      const bool fresh = m_run == -INFINITY;
+      float mk = fresh ? 0.f : m_run * p.kappa;
 #pragma unroll
-    for (int kvb = 0; kvb < KVB; ++kvb)
+      for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float e = __builtin_amdgcn_exp2f(s[kvb][v] * p.kappa - mk);
-        s[kvb][v] = e;
-        rs += e;
+        for (int v = 0; v < 16; ++v) {
+          e[kvb][v] = __builtin_amdgcn_exp2f(s[kvb][v] * p.kappa - mk);
+          rs += e[kvb][v];
+        }
+      if (__builtin_amdgcn_ballot_w64(fresh || !(rs <= kRescaleLimit)) != 0) {  // wave-uniform, rare
+        float x = s[0][0];
+#pragma unroll
+        for (int kvb = 0; kvb < KVB; ++kvb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) x = fmaxf(x, s[kvb][v]);
+        const float m_new = fmaxf(m_run, pair_max(x));
+        // a row with no visible key so far keeps m = -inf; exp2 of (-inf - -inf) is avoided
+        const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * p.kappa);
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DVB; ++i)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+        mk = (m_run == -INFINITY) ? 0.f : m_run * p.kappa;
+        rs = 0.f;
+#pragma unroll
+        for (int kvb = 0; kvb < KVB; ++kvb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            e[kvb][v] = __builtin_amdgcn_exp2f(s[kvb][v] * p.kappa - mk);
+            rs += e[kvb][v];
+          }
       }
+    } else {
+      // the 256-row kernels for 192-feature keys have no registers for a second score tile: tile maximum first
+      float x = s[0][0];
+#pragma unroll
+      for (int kvb = 0; kvb < KVB; ++kvb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x = fmaxf(x, s[kvb][v]);
+      const float mx = pair_max(x);
+      const bool refresh = (mx - m_run) * p.kappa > kRescaleThreshold;  // true on the first tile (m = -inf)
+      if (__builtin_amdgcn_ballot_w64(refresh) != 0) {                   // wave-uniform
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * p.kappa);
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DVB; ++i)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+      }
+      const float mk = (m_run == -INFINITY) ? 0.f : m_run * p.kappa;
+#pragma unroll
+      for (int kvb = 0; kvb < KVB; ++kvb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          e[kvb][v] = __builtin_amdgcn_exp2f(s[kvb][v] * p.kappa - mk);
+          rs += e[kvb][v];
+        }
+    }
     l_run += rs;
 #pragma unroll
     for (int kvb = 0; kvb < KVB; ++kvb)
 #pragma unroll
       for (int jj = 0; jj < 2; ++jj) {
-        const f32x16& x16 = s[kvb];
+        const f32x16& x16 = e[kvb];
         pf[2 * kvb + jj] = to_bf16x8(x16[8 * jj], x16[8 * jj + 1], x16[8 * jj + 2], x16[8 * jj + 3], x16[8 * jj + 4],
                                      x16[8 * jj + 5], x16[8 * jj + 6], x16[8 * jj + 7]);
       }
@@ -232,8 +282,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
     for (int j = 0; j < 2 * KVB; ++j)
 #pragma unroll
       for (int i = 0; i < DVB; ++i) {
-        const bf16x8 a = lds_read_transposed_at(vtile + v_off[i][0] + j * 16 * kRowBytes128,
-                                                vtile + v_off[i][1] + j * 16 * kRowBytes128);
+        const bf16x8 a = lds_read_transposed_at(vtile + v_off(i, 0) + j * 16 * kRowBytes128,
+                                                vtile + v_off(i, 1) + j * 16 * kRowBytes128);
         oacc[i] = mfma32(a, pf[j], oacc[i]);
       }
   };
@@ -243,13 +293,14 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   auto matrix_block = [&](const char* vtile, const char* ktile) __attribute__((always_inline)) {
     constexpr int NPV = 2 * KVB * DVB, NQK = KVB * KS;
     static_assert(kAhead <= NPV, "look-ahead assumes it starts inside the P V product");
+    __builtin_amdgcn_s_setprio(2);  // the wave that owns the matrix pipe issues first
     bf16x8 av[2 * KVB][DVB], ak[KS][KVB];
 #pragma unroll
     for (int j = 0; j < 2 * KVB; ++j)
 #pragma unroll
       for (int i = 0; i < DVB; ++i)
-        av[j][i] = lds_read_transposed_at(vtile + v_off[i][0] + j * 16 * kRowBytes128,
-                                          vtile + v_off[i][1] + j * 16 * kRowBytes128);
+        av[j][i] = lds_read_transposed_at(vtile + v_off(i, 0) + j * 16 * kRowBytes128,
+                                          vtile + v_off(i, 1) + j * 16 * kRowBytes128);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -279,6 +330,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(0);
   };
 
   // Every interval ends by waiting until at most the loads of the last kDist - 1 intervals are
@@ -303,6 +356,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
     constexpr bool LATE = decltype(late_tag)::value, FULL = decltype(full_tag)::value;
     const char* vtile = vbuf + (i & (kSlots - 1)) * kTile;
     const char* ktile = kbuf + ((i + 1) & (kSlots - 1)) * kKTile;
+    refresh_offsets();
     const bool steady = i + 1 + kDist < n_tiles_wg;  // both a K and a V tile are requested in this interval
     // Requests are placed where no LDS read of the same wave follows closely: after the matrix
     // block in the early waves, before the vector block in the late ones.
@@ -382,6 +436,33 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   float* lse = p.lse + b * p.lse_bs + (int64_t)h * p.lse_hs;
   const float l = pair_sum(l_run);
   const float inv = l > 0.f ? 1.f / l : 0.f;
+  if constexpr (!CAUSAL) {
+    if (p.prev_o != nullptr) {  // the same for the whole launch
+      // ---- merging epilogue: the ring's log2-domain online-softmax combine of this chunk's (O, LSE2) with the running
+      // (prev_o, lse) of the rows: M = max(l1, l2), w = 2^(l - M), out = (w1 o1 + w2 o2) / (w1 + w2),
+      // lse = M + log2(w1 + w2). The chunk's O is acc / l, so its weight and 1 / l fold into one factor per row.
+      const float lse_new = l > 0.f ? __builtin_amdgcn_logf(l) + m_run * p.kappa : -INFINITY;
+      const float lse_old = qrow < p.Sq ? lse[qrow] : -INFINITY;
+      const float big = fmaxf(lse_old, lse_new);
+      // both sides empty (-inf): weights 0, result (0, -inf); the ring never gets there (it starts from finfo.min)
+      const float w_old = big == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lse_old - big);
+      const float w_new = big == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lse_new - big);
+      const float den = w_old + w_new;
+      const float rden = den > 0.f ? 1.f / den : 0.f;
+      char* const turn = smem + (HALF ? (wave & 3) : wave) * kRowsViaLdsBytes<DVB>;
+      const int64_t prev_rs = o_row_stride;  // the three tensors share the [.., Hq, 128] row layout
+      const char* prev = reinterpret_cast<const char*>(p.prev_o) +
+                         (b * p.prev_bs + (int64_t)h * kDv + q_wave0 * prev_rs) * (p.prev_f32 ? 4 : 2);
+      // which of the two outputs this wave's 32 rows go to (the ranges lie on multiples of 32 rows)
+      const bool to_o = p.o && q_wave0 >= p.o_r0 && q_wave0 < p.o_r1;
+      const bool to_acc = p.acc_o && q_wave0 >= p.acc_r0 && q_wave0 < p.acc_r1;
+      merge_rows32_via_lds<DVB>(turn, prev, p.prev_f32 != 0, prev_rs, to_o ? oh + q_wave0 * o_row_stride : nullptr, o_row_stride,
+                                to_acc ? p.acc_o + b * p.acc_bs + (int64_t)h * kDv + q_wave0 * o_row_stride : nullptr,
+                                o_row_stride, p.Sq - q_wave0, oacc, w_new * inv * rden, w_old * rden, lane);
+      if (qrow < p.Sq && g == 0) lse[qrow] = den > 0.f ? big + __builtin_amdgcn_logf(den) : -INFINITY;
+      return;
+    }
+  }
   // O^T sits in the accumulators (a lane owns one query row): turned through LDS so that the stores
   // cover whole rows. Every wave is past the barrier behind the last tile read (HALF: past the merge).
   // (Not in the 256-row causal kernel for 192-feature keys, which has no register to spare: the extra

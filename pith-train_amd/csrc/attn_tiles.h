@@ -361,4 +361,65 @@ __device__ __forceinline__ void store_rows32_via_lds(char* lds, OutT* block, int
   }
 }
 
+// The same turn through LDS for the forward kernel's merging epilogue: row r of the block becomes
+//     f_new[r] * accT[r] + f_old[r] * prev[r]
+// (the online-softmax combine of the chunk result in the accumulators with the running result `prev`, bf16 or fp32,
+// whose per-row weights the caller has formed from the two LSEs) and is written as bf16 to `out_bf16` and / or as fp32
+// to `out_f32` (either may be null, either may alias `prev`: a lane reads the old values of a piece before it writes
+// that piece, and no other lane touches it). f_new / f_old are this lane's (= this row's) weights; the old weight
+// travels to the lanes that handle the row's pieces through the 16 bytes of padding behind the row in LDS.
+// All three tensors are addressed from row 0 of the block, feature 0 of the head.
+template <int NB>
+__device__ __forceinline__ void merge_rows32_via_lds(char* lds, const void* prev, bool prev_f32, int64_t prev_row_stride,
+                                                     __bf16* out_bf16, int64_t out_row_stride, float* out_f32,
+                                                     int64_t acc_row_stride, int rows_valid, const f32x16 (&accT)[NB],
+                                                     float f_new, float f_old, int lane) {
+  constexpr int kPitch = NB * 128 + 16;
+  constexpr int kPieces = NB * 8;
+  constexpr int kIters = 32 * kPieces / 64;
+  if (rows_valid <= 0) return;  // wave-uniform
+  const int c = lane & 31, g = lane >> 5;
+  // the running values first: their memory latency then overlaps the turn through LDS (the accumulators are still
+  // live, which the epilogue can afford)
+  f32x4 old[kIters];
+  int row[kIters], piece[kIters];
+#pragma unroll
+  for (int it = 0; it < kIters; ++it) {
+    const int idx = it * 64 + lane;
+    row[it] = idx / kPieces;
+    piece[it] = idx - row[it] * kPieces;
+    const int src_row = row[it] < rows_valid ? row[it] : 0;
+    if (prev_f32) {
+      old[it] = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(prev) + src_row * prev_row_stride + 4 * piece[it]);
+    } else {
+      const u32x2 w = *reinterpret_cast<const u32x2*>(reinterpret_cast<const __bf16*>(prev) + src_row * prev_row_stride + 4 * piece[it]);
+      old[it] = f32x4{bf16lo_to_f32(w[0]), bf16hi_to_f32(w[0]), bf16lo_to_f32(w[1]), bf16hi_to_f32(w[1])};
+    }
+  }
+#pragma unroll
+  for (int o = 0; o < NB; ++o)
+#pragma unroll
+    for (int b4 = 0; b4 < 4; ++b4) {
+      const f32x4 x = {accT[o][4 * b4] * f_new, accT[o][4 * b4 + 1] * f_new, accT[o][4 * b4 + 2] * f_new,
+                       accT[o][4 * b4 + 3] * f_new};
+      *reinterpret_cast<f32x4*>(lds + c * kPitch + (32 * o + 8 * b4 + 4 * g) * 4) = x;
+    }
+  if (g == 0) *reinterpret_cast<float*>(lds + c * kPitch + NB * 128) = f_old;
+  // the reads below see the writes above: one wave's LDS operations execute in order
+#pragma unroll
+  for (int it = 0; it < kIters; ++it) {
+    const f32x4 val = *reinterpret_cast<const f32x4*>(lds + row[it] * kPitch + piece[it] * 16);
+    const float fo = *reinterpret_cast<const float*>(lds + row[it] * kPitch + NB * 128);
+    if (row[it] >= rows_valid) continue;
+    const f32x4 r = val + old[it] * fo;
+    if (out_f32) *reinterpret_cast<f32x4*>(out_f32 + row[it] * acc_row_stride + 4 * piece[it]) = r;
+    if (out_bf16) {
+      u32x2 w;
+      w[0] = pack_bf16x2(r[0], r[1]);
+      w[1] = pack_bf16x2(r[2], r[3]);
+      *reinterpret_cast<u32x2*>(out_bf16 + row[it] * out_row_stride + 4 * piece[it]) = w;
+    }
+  }
+}
+
 }  // namespace pith

@@ -55,6 +55,9 @@ class AttnFwdArgs(Structure):
         ("lse_bs", c_int64), ("lse_hs", c_int64),
         ("scale", c_float), ("causal", c_int32),
         ("k_pe", c_void_p), ("k_pe_bs", c_int64), ("k_pe_rs", c_int64),
+        ("prev_o", c_void_p), ("prev_o_bs", c_int64), ("acc_o", c_void_p), ("acc_o_bs", c_int64),
+        ("prev_o_dtype", c_int32), ("reserved0", c_int32),
+        ("o_rows", c_int64 * 2), ("acc_o_rows", c_int64 * 2),
     ]  # fmt: skip
 
 

@@ -67,30 +67,59 @@ def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool, 
         assert q.shape[1] == k.shape[1], "causal attention needs equal query and key lengths"
 
 
+MERGING_HEAD_DIMS = ((128, 128), (192, 128))  # forward kernels that can merge with a running result
+
+
 def attn_fwd_into(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
     softmax_scale: float, causal: bool, k_pe: torch.Tensor = None,
+    prev_o: torch.Tensor = None, acc_o: torch.Tensor = None, o_rows=None, acc_o_rows=None,
 ) -> None:  # fmt: skip
     """o, lse <- attention(q, k, v). o [b, sq, hq, dv] bf16 and lse [b, hq, sq] fp32 are written.
 
     With k_pe ([b, skv, 64], the MLA layer's rotary key part, one vector per position shared by all
     heads) k is the 128-feature k_nope and the key of head h is [k[:, :, h] | k_pe]: what
-    pithtrain/models/deepseek_v2_lite.py:448-454 materialises is read in place instead."""
+    pithtrain/models/deepseek_v2_lite.py:448-454 materialises is read in place instead.
+
+    With prev_o (bf16 or fp32, shaped like o) the call is a whole ring step: the chunk's result is merged in
+    the kernel's epilogue with the running (prev_o, lse) as _online_softmax_combine_log2 would merge them
+    (pithtrain/operators/ring_attention/mla.py:27-40); lse is read and overwritten, the merged output goes to
+    o (bf16; may be None) and / or acc_o (fp32; may be None); either may be prev_o itself. o_rows / acc_o_rows
+    ((begin, end) query rows of this call on multiples of 32, None = all) restrict which rows each output
+    receives. Head dims in MERGING_HEAD_DIMS, causal=False only."""
     _check_qkv(q, k, v, causal, k_pe)
-    _C.require_device(q, o, lse)
+    _C.require_device(q, lse)
     b, sq, hq, d_q = q.shape
     _, skv, hkv, d_v = v.shape
-    assert o.dtype == torch.bfloat16 and tuple(o.shape) == (b, sq, hq, d_v), "o has the wrong dtype or shape"
     assert lse.dtype == torch.float32 and tuple(lse.shape) == (b, hq, sq), "lse has the wrong dtype or shape"
     lse_bs, lse_hs = _C.bhs_strides(lse, "lse")
     args = _C.AttnFwdArgs(
-        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), o=o.data_ptr(), lse=lse.data_ptr(),
+        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), o=None, lse=lse.data_ptr(),
         B=b, Sq=sq, Skv=skv, Hq=hq, Hkv=hkv, Dqk=d_q, Dv=d_v,
         q_bs=_C.bshd_batch_stride(q, "q"), k_bs=_C.bshd_batch_stride(k, "k"),
-        v_bs=_C.bshd_batch_stride(v, "v"), o_bs=_C.bshd_batch_stride(o, "o"),
+        v_bs=_C.bshd_batch_stride(v, "v"), o_bs=0,
         lse_bs=lse_bs, lse_hs=lse_hs, scale=float(softmax_scale), causal=int(bool(causal)),
         k_pe=None, k_pe_bs=0, k_pe_rs=0,
     )  # fmt: skip
+    if o is not None:
+        _C.require_device(q, o)
+        assert o.dtype == torch.bfloat16 and tuple(o.shape) == (b, sq, hq, d_v), "o has the wrong dtype or shape"
+        args.o, args.o_bs = o.data_ptr(), _C.bshd_batch_stride(o, "o")
+    if prev_o is not None:
+        _C.require_device(q, prev_o)
+        assert tuple(prev_o.shape) == (b, sq, hq, d_v), "prev_o has the wrong shape"
+        assert o is not None or acc_o is not None, "a merging call needs o or acc_o"
+        args.prev_o, args.prev_o_bs, args.prev_o_dtype = prev_o.data_ptr(), _C.bshd_batch_stride(prev_o, "prev_o"), _C.dtype_code(prev_o)
+        if acc_o is not None:
+            _C.require_device(q, acc_o)
+            assert acc_o.dtype == torch.float32 and tuple(acc_o.shape) == (b, sq, hq, d_v), "acc_o has the wrong dtype or shape"
+            args.acc_o, args.acc_o_bs = acc_o.data_ptr(), _C.bshd_batch_stride(acc_o, "acc_o")
+        if o_rows is not None:
+            args.o_rows[0], args.o_rows[1] = o_rows
+        if acc_o_rows is not None:
+            args.acc_o_rows[0], args.acc_o_rows[1] = acc_o_rows
+    else:
+        assert o is not None and acc_o is None, "o is required (and acc_o unused) without prev_o"
     if k_pe is not None:
         k_pe, args.k_pe_bs, args.k_pe_rs = _k_pe_strides(k, k_pe)
         args.k_pe = k_pe.data_ptr()

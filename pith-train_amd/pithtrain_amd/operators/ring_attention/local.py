@@ -42,6 +42,7 @@ import torch
 
 from pithtrain_amd import _C
 from pithtrain_amd.operators.mla.hip import (
+    MERGING_HEAD_DIMS,
     attn_bwd_delta_into,
     attn_bwd_pair_into,
     attn_fwd_into,
@@ -49,6 +50,9 @@ from pithtrain_amd.operators.mla.hip import (
 from pithtrain_amd.operators.ring_attention.combine import cast_f32_bf16_into, combine_into
 
 LAYOUTS = ("contiguous", "zigzag")
+# Ring steps after the first merge inside the forward kernel (one launch per step) where the kernels support it;
+# False restores chunk forward + combine launch per step (kept for comparison runs).
+FUSE_MERGE = True
 
 
 @dataclass(frozen=True)
@@ -159,11 +163,20 @@ class RingForward:
         self.acc = None
         if any(n > 1 for n in self.pending.values()):
             self.acc = torch.empty((B, S, H, dv_dim), dtype=torch.float32, device=q.device)
+        # Steps after the first merge into the running state inside the forward kernel's epilogue where the
+        # kernels for these head dims can (fuse_merge); otherwise the chunk result goes to step_out / step_lse
+        # and a combine launch merges it.
+        self.fuse_merge = FUSE_MERGE and (q.shape[-1], dv_dim) in MERGING_HEAD_DIMS
+        self.dv_dim = dv_dim
         self.step_out = self.step_lse = None
-        if len(self.steps) > 1:
-            self.step_out = torch.empty((B, S, H, dv_dim), dtype=torch.bfloat16, device=q.device)
-            self.step_lse = torch.empty(B * H * S, dtype=torch.float32, device=q.device)
         self.done = 0
+
+    def _step_buffers(self):
+        if self.step_out is None:
+            B, S, H, _ = self.q.shape
+            self.step_out = torch.empty((B, S, H, self.dv_dim), dtype=torch.bfloat16, device=self.q.device)
+            self.step_lse = torch.empty(B * H * S, dtype=torch.float32, device=self.q.device)
+        return self.step_out, self.step_lse
 
     @staticmethod
     def _covers(step: RingStep, r: Tuple[int, int]) -> bool:
@@ -181,9 +194,35 @@ class RingForward:
             assert st.causal and st.q_rows == (0, S)
             attn_fwd_into(self.q, k_j, v_j, self.out, self.lse, self.scale, True, k_pe_j)
             return
+        covered = [r for r in self.ranges if self._covers(st, r)]
+        assert covered and (covered[0][0], covered[-1][1]) == st.q_rows, "a step's query rows must be whole row ranges"
+        if self.fuse_merge and len({self.in_acc[r] for r in covered}) == 1:
+            # One launch: chunk attention + merge. The running value of all covered ranges sits in the same tensor
+            # (the schedule merges them equally often up to here); ranges that are merged again later get the fp32
+            # result, ranges whose last merge this is get bf16. A launch that covers both kinds tells the kernel
+            # which rows go where when the boundaries allow it (multiples of 32 rows); otherwise it writes both
+            # outputs for every row, and the surplus rows of either tensor are overwritten later or never read.
+            prev = self.acc if self.in_acc[covered[0]] else self.out
+            last = [r for r in covered if self.pending[r] == 1]
+            more = [r for r in covered if self.pending[r] > 1]
+            o_rows = acc_rows = None
+            if last and more:
+                spans = [(rs[0][0] - st.q_rows[0], rs[-1][1] - st.q_rows[0]) for rs in (last, more)]
+                whole = all(sum(r[1] - r[0] for r in rs) == sp[1] - sp[0] for rs, sp in zip((last, more), spans))
+                if whole and all(sp[0] % 32 == 0 and (sp[1] % 32 == 0 or sp[1] == st.q_rows[1] - st.q_rows[0]) for sp in spans):
+                    o_rows, acc_rows = spans
+            attn_fwd_into(_rows(self.q, st.q_rows), _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows),
+                          _rows(self.out, st.q_rows) if last else None, _lse_rows(self.lse, st.q_rows), self.scale, False,
+                          _pe_rows(k_pe_j, st.kv_rows), prev_o=_rows(prev, st.q_rows),
+                          acc_o=_rows(self.acc, st.q_rows) if more else None, o_rows=o_rows, acc_o_rows=acc_rows)  # fmt: skip
+            for r in covered:
+                self.pending[r] -= 1
+                self.in_acc[r] = self.pending[r] > 0
+            return
         n_q = st.q_rows[1] - st.q_rows[0]
-        so = self.step_out[:, :n_q]
-        sl = self.step_lse[: B * H * n_q].view(B, H, n_q)
+        step_out, step_lse = self._step_buffers()
+        so = step_out[:, :n_q]
+        sl = step_lse[: B * H * n_q].view(B, H, n_q)
         attn_fwd_into(_rows(self.q, st.q_rows), _rows(k_j, st.kv_rows), _rows(v_j, st.kv_rows), so, sl,
                       self.scale, False, _pe_rows(k_pe_j, st.kv_rows))  # fmt: skip
         # Ranges in the same state are merged by one launch.

@@ -260,3 +260,34 @@ def test_error_is_within_twice_an_eager_bf16_restatement(gpu, causal):
     for name in ours:
         e_ours, e_eager = norm_max_err(ours[name], want[name]), norm_max_err(eager[name], want[name])
         assert e_ours <= 2 * e_eager + 1e-4, f"{name}: error {e_ours:.3e} against {e_eager:.3e} of the eager restatement"
+
+
+@pytest.mark.parametrize("Dqk,Hq,Hkv,Sq,causal", [
+    (128, 8, 2, 512, False), (128, 8, 2, 512, True), (128, 32, 4, 2048, False),  # 128-row and 256-row workgroups
+    (192, 4, 4, 384, True), (192, 48, 48, 1024, False), (64, 4, 2, 320, True),
+])  # fmt: skip
+@pytest.mark.parametrize("ramp", ["climbing", "huge-jump", "falling"])
+def test_forward_when_the_running_maximum_moves(gpu, Dqk, Hq, Hkv, Sq, causal, ramp):
+    """The forward refreshes its running row maximum lazily (a stale maximum is kept while no P value exceeds 2^8).
+    Scores that climb from key tile to key tile, that jump by far more than fp32's exponent range allows
+    exp2(kappa * (s - m_stale)) to hold, or that fall (first tile dominates, everything after underflows) must
+    give the same O and LSE2 as the oracle."""
+    Dv = min(Dqk, 128)
+    q, k, v, _ = _inputs(1, Sq, Sq, Hq, Hkv, Dqk, Dv, seed=17)
+    # keys along a direction every query has a positive component on, growing (or shrinking) with the position
+    direction = torch.zeros(Dqk)
+    direction[0] = 1.0
+    q = q.float()
+    q[..., 0] = q[..., 0].abs() + 1.0
+    pos = torch.arange(Sq, dtype=torch.float32) / Sq
+    gain = {"climbing": 60.0 * pos, "huge-jump": 4000.0 * (pos > 0.5).float(), "falling": 300.0 * (1 - pos)}[ramp]
+    k = (k.float() + gain[None, :, None, None] * direction).to(torch.bfloat16)
+    q = q.to(torch.bfloat16)
+    scale = Dqk**-0.5
+    ref_o, ref_lse = R.chunk_fwd(q, k, v, scale, causal)
+    o, lse = _mla_fwd(q.to(gpu), k.to(gpu), v.to(gpu), scale, causal=causal)
+    check_bf16_result(o, ref_o, f"O ({ramp})")
+    # LSE2 is large here (up to thousands): 1e-3 absolute is below fp32 resolution of such values, so the bound is
+    # relative to the magnitude for them
+    err = (lse.double().cpu() - ref_lse).abs()
+    assert (err <= 1e-3 + 2e-7 * ref_lse.abs()).all(), f"LSE2 ({ramp}): max error {err.max().item():.3e}"

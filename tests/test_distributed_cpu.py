@@ -22,9 +22,14 @@ def _install_cpu_stand_ins():
     def full_key(k, k_pe):  # keys in two parts: [k_nope | k_pe for every head]
         return k if k_pe is None else torch.cat([k, k_pe.unsqueeze(2).expand(-1, -1, k.shape[2], -1)], -1)
 
-    def attn_fwd_into(q, k, v, o, lse, scale, causal, k_pe=None):
+    def attn_fwd_into(q, k, v, o, lse, scale, causal, k_pe=None, prev_o=None, acc_o=None):
         ro, rl = R.chunk_fwd(q, full_key(k, k_pe), v, scale, causal)
-        o.copy_(ro)
+        if prev_o is not None:  # the merging form: one ring step
+            ro, rl = R.combine_log2(prev_o.double(), lse.double(), ro, rl)
+        if o is not None:
+            o.copy_(ro)
+        if acc_o is not None:
+            acc_o.copy_(ro)
         lse.copy_(rl)
 
     def attn_bwd_delta_into(out, dout, delta):

@@ -334,16 +334,6 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
     __builtin_amdgcn_s_setprio(0);
   };
 
-  // Every interval ends by waiting until at most the loads of the last kDist - 1 intervals are
-  // still in flight (the tiles of the next interval have landed), and a workgroup barrier.
-  constexpr int kPerInterval = 2 * DirectTile128<kBN, kThreads>::kPerThread + (DQK == 192 ? 1 : 0);
-  static_assert((kDist - 1) * kPerInterval < 16, "vmcnt immediate below assumes a 4-bit low field");
-  auto land_and_sync = [&](bool steady) __attribute__((always_inline)) {
-    if (steady) __builtin_amdgcn_s_waitcnt(0x0F70 | ((kDist - 1) * kPerInterval));
-    else __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-  };
-
   // ---- prologue: S(0) (and P(0) in the early waves) from K tile 0
   __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far, Q fragments included
   __syncthreads();
@@ -352,17 +342,28 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   if (!late) softmax(0);
 
   // One interval; FULL: this wave has both a tile to accumulate and a next tile to score.
-  auto interval = [&](int i, auto late_tag, auto full_tag) __attribute__((always_inline)) {
+  // Intervals come in pairs (even, odd): the even one requests the tiles of BOTH intervals of the pair after next
+  // (K i+3, i+4 and V i+2, i+3), the odd one ends with the wait for those loads and the workgroup barrier. A slot
+  // that is refilled was last read before the barrier that precedes the request, and everything an interval reads
+  // had landed before the barrier that precedes the pair. PAIR: 1 = even, 2 = odd, 0 = decided from i at run time.
+  auto interval = [&](int i, auto late_tag, auto full_tag, auto pair_tag) __attribute__((always_inline)) {
     constexpr bool LATE = decltype(late_tag)::value, FULL = decltype(full_tag)::value;
+    constexpr int PAIR = decltype(pair_tag)::value;
+    const bool even = PAIR == 1 || (PAIR == 0 && !(i & 1));
     const char* vtile = vbuf + (i & (kSlots - 1)) * kTile;
     const char* ktile = kbuf + ((i + 1) & (kSlots - 1)) * kKTile;
     refresh_offsets();
-    const bool steady = i + 1 + kDist < n_tiles_wg;  // both a K and a V tile are requested in this interval
     // Requests are placed where no LDS read of the same wave follows closely: after the matrix
     // block in the early waves, before the vector block in the late ones.
     auto request = [&]() __attribute__((always_inline)) {
-      if (i + 1 + kDist < n_tiles_wg) issue_k(i + 1 + kDist);
-      if (i + kDist < n_tiles_wg) issue_v(i + kDist);
+      if constexpr (PAIR != 2) {
+        if (even) {
+          if (i + 3 < n_tiles_wg) issue_k(i + 3);
+          if (i + 2 < n_tiles_wg) issue_v(i + 2);
+          if (i + 4 < n_tiles_wg) issue_k(i + 4);
+          if (i + 3 < n_tiles_wg) issue_v(i + 3);
+        }
+      }
     };
     if (!LATE) {
       if (FULL) {
@@ -381,19 +382,30 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
       if (FULL) matrix_block(vtile, ktile);
       else if (i < n_tiles_wave) accumulate(vtile);
     }
-    land_and_sync(steady);
+    if (PAIR == 2 || !even || i + 1 == n_tiles_wg) {  // the same decision in every wave of the workgroup
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+    }
   };
   // Every wave passes the same number of barriers; the two roles run separate loops so that
   // each loop body is straight-line code around one accumulator set.
-  if (!late) {
+  auto run = [&](auto late_tag) __attribute__((always_inline)) {
+    using Full = std::true_type;
+    using Part = std::false_type;
     int i = 0;
-    for (; i + 1 < n_tiles_wave; ++i) interval(i, std::false_type{}, std::true_type{});
-    for (; i < n_tiles_wg; ++i) interval(i, std::false_type{}, std::false_type{});
-  } else {
-    int i = 0;
-    for (; i + 1 < n_tiles_wave; ++i) interval(i, std::true_type{}, std::true_type{});
-    for (; i < n_tiles_wg; ++i) interval(i, std::true_type{}, std::false_type{});
-  }
+    // the pair as one loop body (no parity tests, the odd interval without request code) wherever two copies of the
+    // interval still fit the registers
+    if constexpr (!(DQK == 192 && !HALF)) {
+      for (; i + 2 < n_tiles_wave; i += 2) {
+        interval(i, late_tag, Full{}, std::integral_constant<int, 1>{});
+        interval(i + 1, late_tag, Full{}, std::integral_constant<int, 2>{});
+      }
+    }
+    for (; i + 1 < n_tiles_wave; ++i) interval(i, late_tag, Full{}, std::integral_constant<int, 0>{});
+    for (; i < n_tiles_wg; ++i) interval(i, late_tag, Part{}, std::integral_constant<int, 0>{});
+  };
+  if (!late) run(std::false_type{});
+  else run(std::true_type{});
 
   // ---- HALF: the late wave of a pair hands its accumulator, maximum and sum to the early wave,
   // which rescales both to the common maximum and adds them. The tile ring is free by now (every

@@ -196,7 +196,18 @@ int pith_attn_bwd_delta(const pith_attn_delta_args* args, pith_stream_t stream);
  * (kv_row_heads*D) elements, and lse / delta are addressed through their head stride as always.
  * Results equal the corresponding heads of a call on all heads. This is how a caller bounds the
  * dS hand-over buffer below: one kv head (and its query heads) at a time through one small buffer.
- * Not available together with k_pe. */
+ * Not available together with k_pe.
+ *
+ * Two ring conveniences that save separate launches (no counterpart in the reference, which runs
+ * `torch.zeros_like` per step and adds bf16 partial dQ, standard.py:131-133, mla.py:103,116):
+ *   dkv_zero_tail: pith_attn_bwd_dkdv also sets rows [Skv, Skv + dkv_zero_tail) of dk and dv to
+ *     zero (not dk_pe; ignored with accumulate_dkv): the rows of a chunk that a zigzag step does not
+ *     see owe a zero gradient.
+ *   dq_final (pith_attn_bwd_dq, dq_dtype PITH_F32, head dims (128,128)): query rows
+ *     [dq_final_rows[0], dq_final_rows[1]) (multiples of 32 or Sq; {0,0} = all) receive their
+ *     result - the old contents of dq included when accumulate_dq is set - rounded to bf16 in
+ *     dq_final [B,Sq,Hq,Dqk] (laid out like dq) instead of dq: the last ring step that touches a row
+ *     range emits the final bf16 gradient, and no cast pass over the fp32 accumulator is needed. */
 typedef struct {
   const void* q;
   const void* k;
@@ -225,6 +236,10 @@ typedef struct {
   int64_t ds_bytes;          /* its size */
   int64_t q_row_heads;       /* heads per row of q, dout, dq (0 = Hq) */
   int64_t kv_row_heads;      /* heads per row of k, v, dk, dv (0 = Hkv) */
+  int64_t dkv_zero_tail;     /* rows behind the Skv rows of dk, dv to clear (0 = none) */
+  void* dq_final;            /* bf16 destination of finished dQ rows, or NULL */
+  int64_t dq_final_bs;       /* its batch stride, elements */
+  int64_t dq_final_rows[2];  /* query rows that go to dq_final ({0,0} = all) */
 } pith_attn_bwd_args;
 
 int pith_attn_bwd_dkdv(const pith_attn_bwd_args* args, pith_stream_t stream);

@@ -40,7 +40,41 @@ struct BwdParams {
   char* ds;
   int ds_qt, ds_kb;
   int64_t ds_hs;
+  // dQ kernels, fp32 dq: query rows [final_r0, final_r1) (multiples of 32, or Sq) receive their result, old
+  // contents of dq included when accumulating, as bf16 in dq_final instead of dq (nullptr: none do)
+  __bf16* dq_final;
+  int64_t dq_final_bs;
+  int final_r0, final_r1;
+  // dK/dV kernels: blocks main_blocks .. of the grid clear rows [Skv, Skv + zero_tail) of dk and dv
+  int zero_tail, main_blocks;
 };
+
+constexpr int kZeroTailRows = 32;  // rows one such block clears
+
+// The body of a dK/dV workgroup beyond the main grid: zero-fills its share of the rows behind the Skv rows the
+// call computes (a ring step that sees only the first rows of a chunk owes the others a zero gradient).
+// dk_feats: features per head of dk (128 when the keys come in two parts).
+template <typename OutT>
+__device__ __forceinline__ void zero_tail_block(const BwdParams& p, int idx, int dk_feats, int dv_feats, int tid, int threads) {
+  const int r0 = p.Skv + idx * kZeroTailRows;
+  const int rows = min(kZeroTailRows, p.Skv + p.zero_tail - r0);
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  constexpr int kPer16 = 16 / (int)sizeof(OutT);  // elements per 16-byte piece
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    OutT* base = reinterpret_cast<OutT*>(t == 0 ? p.dk : p.dv);
+    const int64_t bs = t == 0 ? p.dk_bs : p.dv_bs;
+    const int feats = t == 0 ? dk_feats : dv_feats;
+    const int64_t row_stride = (int64_t)p.HkvT * feats;  // a row holds HkvT heads, Hkv of them belong to this call
+    const int pieces = p.Hkv * feats / kPer16;
+    const int total = p.B * rows * pieces;
+    for (int i = tid; i < total; i += threads) {
+      const int piece = i % pieces, rb = i / pieces;
+      const int row = r0 + rb % rows, b = rb / rows;
+      *reinterpret_cast<u32x4*>(base + b * bs + row * row_stride + (int64_t)piece * kPer16) = zero;
+    }
+  }
+}
 
 constexpr int kDsBlockBytes = 4 * 4096;  // one (query tile, key block): four wave-pair images
 // Number of 16 KB blocks that precede query tile t within a head.
@@ -84,9 +118,11 @@ __device__ __forceinline__ void store4<__bf16>(__bf16* dst, float a0, float a1, 
 // the block; rows at or beyond `rows_valid` are skipped. With `accumulate` the old values of a batch of rows are all read before
 // the batch's first store (row pointers may alias as far as the compiler can tell; it would chain load - store - load
 // otherwise).
+// With `final_block` (wave-uniform; the same rows of a bf16 tensor laid out like `block`) the result, old values included,
+// is rounded to bf16 and written there, and `block` keeps what it held.
 template <typename OutT, int NB>
 __device__ __forceinline__ void store_rows32(OutT* block, int64_t row_stride, int rows_valid, const f32x16 (&acc)[NB],
-                                             float factor, bool accumulate, int c, int g) {
+                                             float factor, bool accumulate, int c, int g, __bf16* final_block = nullptr) {
 #pragma clang fp contract(off)  // product rounded, then added: what accumulating into a separate tensor gives
   constexpr int kBatch = NB > 4 ? 4 : 8;  // accumulator elements per lane and batch: NB * kBatch old values in registers
   // a block wholly beyond the last row (wave-uniform): `block` itself is out of range, so not even the clamped
@@ -109,11 +145,13 @@ __device__ __forceinline__ void store_rows32(OutT* block, int64_t row_stride, in
       const int r = acc_row(v0 + dv, g);
       if (r < rows_valid) {
         OutT* dst = block + r * row_stride + c;
+        __bf16* fin = final_block + r * row_stride + c;
 #pragma unroll
         for (int o = 0; o < NB; ++o) {
           float x = acc[o][v0 + dv] * factor;
           if (accumulate) x += old[dv][o];
-          dst[32 * o] = (OutT)x;
+          if (final_block != nullptr) fin[32 * o] = (__bf16)x;
+          else dst[32 * o] = (OutT)x;
         }
       }
     }

@@ -151,6 +151,10 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
   __shared__ __attribute__((aligned(16))) char smem[L::kTotal];
 
   const int tid = threadIdx.x;
+  if ((int)blockIdx.x >= p.main_blocks) {  // workgroups appended to the grid: clear the rows behind the chunk's visible part
+    zero_tail_block<OutT>(p, (int)blockIdx.x - p.main_blocks, DQK, DV, tid, kThreads);
+    return;
+  }
   const int lane = tid & 63, wave = tid >> 6;
   const int c = lane & 31, g = lane >> 5;
   const int pair = wave & 3;
@@ -327,7 +331,9 @@ template <int DQK, int DV>
 void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
   p.tiles = (int)((a->Skv + kBN - 1) / kBN);
   p.accumulate = a->accumulate_dkv;
-  const dim3 grid((unsigned)(p.tiles * a->Hkv * a->B * p.split)), block(kThreads);
+  p.main_blocks = (int)(p.tiles * a->Hkv * a->B * p.split);
+  p.zero_tail = a->accumulate_dkv ? 0 : (int)a->dkv_zero_tail;  // rows that are added to keep what they hold
+  const dim3 grid((unsigned)(p.main_blocks + (p.zero_tail + kZeroTailRows - 1) / kZeroTailRows)), block(kThreads);
   const bool f32 = a->dkv_dtype == PITH_F32;
   if constexpr (DQK == 128 && DV == 128) {
     launch_dkdv_d128(p, a->causal != 0, f32, grid.x, st);

@@ -67,6 +67,10 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   __shared__ __attribute__((aligned(1024))) char smem[kSmem];
 
   const int tid = threadIdx.x;
+  if ((int)blockIdx.x >= p.main_blocks) {  // workgroups appended to the grid: clear the rows behind the chunk's visible part
+    zero_tail_block<OutT>(p, (int)blockIdx.x - p.main_blocks, kD, kD, tid, kThreads);
+    return;
+  }
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, g = lane >> 5;
   const int pair = wave & 3;

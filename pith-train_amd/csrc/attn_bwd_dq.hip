@@ -250,6 +250,8 @@ int validate_bwd(const pith_attn_bwd_args* a, const char* who, bool need_dq, boo
                 (long long)a->q_row_heads, (long long)a->kv_row_heads, (long long)a->Hq, (long long)a->Hkv);
   if (a->k_pe && (a->q_row_heads > a->Hq || a->kv_row_heads > a->Hkv))
     return fail(PITH_ERR_UNSUPPORTED, "%s: keys in two parts cannot be combined with a head range of wider tensors", who);
+  if (a->dkv_zero_tail < 0 || a->dkv_zero_tail > (1 << 24))
+    return fail(PITH_ERR_BAD_SHAPE, "%s: dkv_zero_tail=%lld out of range", who, (long long)a->dkv_zero_tail);
   if (a->causal && a->Sq != a->Skv)
     return fail(PITH_ERR_UNSUPPORTED, "%s: causal needs Sq == Skv (got %lld, %lld)", who, (long long)a->Sq, (long long)a->Skv);
   if (a->Sq > (1 << 24) || a->Skv > (1 << 24) || a->Hq > 65535 || a->B > 65535 ||
@@ -302,6 +304,8 @@ BwdParams make_bwd_params(const pith_attn_bwd_args* a) {
   p.ds_qt = (int)((a->Sq + 63) / 64);
   p.ds_kb = (int)((a->Skv + kDkdvBlockN - 1) / kDkdvBlockN);
   p.ds_hs = (a->causal ? ds_tile_start<true>(p.ds_qt, p.ds_kb) : ds_tile_start<false>(p.ds_qt, p.ds_kb)) * kDsBlockBytes;
+  p.dq_final = nullptr; p.dq_final_bs = 0; p.final_r0 = p.final_r1 = 0;
+  p.zero_tail = 0; p.main_blocks = 0x7fffffff;
   return p;
 }
 
@@ -322,7 +326,22 @@ extern "C" int64_t pith_attn_bwd_ds_bytes(const pith_attn_bwd_args* a) { return 
 extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t stream) {
   const int rc = validate_bwd(a, "pith_attn_bwd_dq", true, false);
   if (rc != PITH_OK) return rc;
-  const BwdParams p = make_bwd_params(a);
+  BwdParams p = make_bwd_params(a);
+  if (a->dq_final) {
+    if (a->dq_dtype != PITH_F32 || a->Dqk != 128 || a->Dv != 128)
+      return fail(PITH_ERR_UNSUPPORTED, "pith_attn_bwd_dq: dq_final needs an fp32 dq and head dims (128,128)");
+    if (!aligned16(a->dq_final) || a->dq_final_bs % 8)
+      return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_dq: dq_final pointer / batch stride must keep 16-byte alignment");
+    int64_t r0 = a->dq_final_rows[0], r1 = a->dq_final_rows[1];
+    if (r0 == 0 && r1 == 0) r1 = a->Sq;
+    if (r0 < 0 || r1 < r0 || r1 > a->Sq || r0 % 32 || (r1 % 32 && r1 != a->Sq))
+      return fail(PITH_ERR_BAD_SHAPE, "pith_attn_bwd_dq: dq_final_rows = [%lld, %lld) must lie within the %lld query rows on multiples of 32",
+                  (long long)a->dq_final_rows[0], (long long)a->dq_final_rows[1], (long long)a->Sq);
+    p.dq_final = reinterpret_cast<__bf16*>(a->dq_final);
+    p.dq_final_bs = a->dq_final_bs;
+    p.final_r0 = (int)r0;
+    p.final_r1 = (int)r1;
+  }
   hipStream_t st = (hipStream_t)stream;
   begin_launch();
   if (a->ds && ds_bytes_for(a) > 0 && a->ds_bytes >= ds_bytes_for(a)) {

@@ -281,8 +281,11 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_d128_kernel(BwdParams p)
   // hence one more barrier before the rings are overwritten.
   __syncthreads();
   OutT* dqh = reinterpret_cast<OutT*>(p.dq) + b * p.dq_bs + (int64_t)h * kD;
+  __bf16* fin = nullptr;  // rows whose gradient is complete with this call go out as bf16
+  if (p.dq_final != nullptr && q_wave0 >= p.final_r0 && q_wave0 < p.final_r1)
+    fin = p.dq_final + b * p.dq_final_bs + (int64_t)h * kD + q_wave0 * q_row_stride;
   store_rows32_via_lds<OutT, DB>(smem + wave * kRowsViaLdsBytes<DB>, dqh + q_wave0 * q_row_stride, q_row_stride, p.Sq - q_wave0,
-                                 acc, p.scale, p.accumulate != 0, lane);
+                                 acc, p.scale, p.accumulate != 0, lane, fin);
 }
 
 }  // namespace

@@ -434,7 +434,10 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[o][4 * b4 + e] += v4[e];
       }
-    store_rows32_via_lds<OutT, DB>(exch, dqh + q_wave0 * q_row_stride, q_row_stride, p.Sq - q_wave0, acc, p.scale, p.accumulate != 0, lane);
+    __bf16* fin = nullptr;  // rows whose gradient is complete with this call go out as bf16
+    if (p.dq_final != nullptr && q_wave0 >= p.final_r0 && q_wave0 < p.final_r1)
+      fin = p.dq_final + b * p.dq_final_bs + (int64_t)h * DQK + q_wave0 * q_row_stride;
+    store_rows32_via_lds<OutT, DB>(exch, dqh + q_wave0 * q_row_stride, q_row_stride, p.Sq - q_wave0, acc, p.scale, p.accumulate != 0, lane, fin);
   } else if (qrow < p.Sq) {
     OutT* dst = dqh + qrow * q_row_stride;
 #pragma unroll

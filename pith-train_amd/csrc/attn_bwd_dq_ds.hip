@@ -231,7 +231,10 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb) {
     const int row0 = q_wave0 + 32 * rb;
-    store_rows32<OutT, DB>(dqh + row0 * row_stride, row_stride, p.Sq - row0, acc[rb], sc, p.accumulate != 0, c, g);
+    __bf16* fin = nullptr;  // rows whose gradient is complete with this call go out as bf16
+    if (p.dq_final != nullptr && row0 >= p.final_r0 && row0 < p.final_r1)
+      fin = p.dq_final + b * p.dq_final_bs + (int64_t)h * DQK + row0 * row_stride;
+    store_rows32<OutT, DB>(dqh + row0 * row_stride, row_stride, p.Sq - row0, acc[rb], sc, p.accumulate != 0, c, g, fin);
   }
 }
 

@@ -297,13 +297,16 @@ __device__ __forceinline__ bf16x8 lds_read_transposed_at(const char* lo_addr, co
 // instruction at 128 features). `lds` is a wave-private area of kRowsViaLdsBytes<NB> bytes (the tile
 // rings are free by then: the caller has passed the barrier behind their last reader); `factor` is this
 // lane's (= this row's) scale; rows at or beyond rows_valid are neither read nor written (rows_valid may be <= 0).
-// With `accumulate` all old values are read before the first store.
+// With `accumulate` all old values are read before the first store. With `final_block` (wave-uniform; the same rows of
+// a bf16 tensor laid out like `block`) the result, old values included, is rounded to bf16 and written there, and
+// `block` keeps what it held.
 template <int NB>
 constexpr int kRowsViaLdsBytes = 32 * (NB * 128 + 16);
 
 template <typename OutT, int NB>
 __device__ __forceinline__ void store_rows32_via_lds(char* lds, OutT* block, int64_t row_stride, int rows_valid,
-                                                     const f32x16 (&accT)[NB], float factor, bool accumulate, int lane) {
+                                                     const f32x16 (&accT)[NB], float factor, bool accumulate, int lane,
+                                                     __bf16* final_block = nullptr) {
 #pragma clang fp contract(off)  // product rounded, then added: what accumulating into a separate tensor gives
   constexpr int kPitch = NB * 128 + 16;  // bytes; the 16 spread the 32 rows of a column over the banks
   constexpr int kPieces = NB * 8;        // 16-byte pieces (4 features) per row
@@ -344,6 +347,18 @@ __device__ __forceinline__ void store_rows32_via_lds(char* lds, OutT* block, int
         val[it][3] += bf16hi_to_f32(old[1]);
       }
     }
+  }
+  if (final_block != nullptr) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      if (row[it] < rows_valid) {
+        u32x2 w;
+        w[0] = pack_bf16x2(val[it][0], val[it][1]);
+        w[1] = pack_bf16x2(val[it][2], val[it][3]);
+        *reinterpret_cast<u32x2*>(final_block + row[it] * row_stride + 4 * piece[it]) = w;
+      }
+    }
+    return;
   }
 #pragma unroll
   for (int it = 0; it < kIters; ++it) {

@@ -86,6 +86,7 @@ class AttnBwdArgs(Structure):
         ("dk_pe", c_void_p), ("dk_pe_bs", c_int64),
         ("ds", c_void_p), ("ds_bytes", c_int64),
         ("q_row_heads", c_int64), ("kv_row_heads", c_int64),
+        ("dkv_zero_tail", c_int64), ("dq_final", c_void_p), ("dq_final_bs", c_int64), ("dq_final_rows", c_int64 * 2),
     ]  # fmt: skip
 
 

@@ -68,6 +68,7 @@ def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool, 
 
 
 MERGING_HEAD_DIMS = ((128, 128), (192, 128))  # forward kernels that can merge with a running result
+FINAL_DQ_HEAD_DIMS = ((128, 128),)  # dQ kernels that can emit finished rows as bf16 beside an fp32 accumulator
 
 
 def attn_fwd_into(
@@ -264,7 +265,7 @@ def _try_alloc(nbytes: int, device: torch.device):
 def attn_bwd_pair_into(
     q, k, v, dout, lse, delta, dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor, softmax_scale: float, causal: bool,
     accumulate_dq: bool = False, accumulate_dkv: bool = False, k_pe: torch.Tensor = None, dk_pe: torch.Tensor = None,
-    handover: bool = True,
+    handover: bool = True, zero_tail: int = 0, dq_final: torch.Tensor = None, dq_final_rows=None,
 ) -> int:  # fmt: skip
     """Both backward calls of one chunk pair: dk, dv, then dq (see attn_bwd_dkdv_into / attn_bwd_dq_into).
     The dS hand-over between them is decided here (ds_plan), so a buffer can never reach the dQ call without
@@ -274,8 +275,9 @@ def attn_bwd_pair_into(
     hkv = k.shape[2]
     if buf is None or plan[0] == hkv:
         attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, softmax_scale, causal, accumulate=accumulate_dkv,
-                           k_pe=k_pe, dk_pe=dk_pe, ds=buf)  # fmt: skip
-        attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, softmax_scale, causal, accumulate=accumulate_dq, k_pe=k_pe, ds=buf)
+                           k_pe=k_pe, dk_pe=dk_pe, ds=buf, zero_tail=zero_tail)  # fmt: skip
+        attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, softmax_scale, causal, accumulate=accumulate_dq, k_pe=k_pe, ds=buf,
+                         dq_final=dq_final, dq_final_rows=dq_final_rows)  # fmt: skip
         return 0 if buf is None else buf.numel()
     # one group of kv heads after the other, each with its query heads, through the same buffer (the
     # kernels of successive slabs are ordered by the stream)
@@ -284,17 +286,21 @@ def attn_bwd_pair_into(
         kv_h, q_h = slice(h0, h0 + plan[0]), slice(h0 * group, (h0 + plan[0]) * group)
         qs, ds_, ls, dl = q[:, :, q_h], dout[:, :, q_h], lse[:, q_h], delta[:, q_h]
         attn_bwd_dkdv_into(qs, k[:, :, kv_h], v[:, :, kv_h], ds_, ls, dl, dk[:, :, kv_h], dv[:, :, kv_h],
-                           softmax_scale, causal, accumulate=accumulate_dkv, ds=buf)  # fmt: skip
+                           softmax_scale, causal, accumulate=accumulate_dkv, ds=buf, zero_tail=zero_tail)  # fmt: skip
         attn_bwd_dq_into(qs, k[:, :, kv_h], v[:, :, kv_h], ds_, ls, dl, dq[:, :, q_h], softmax_scale, causal,
-                         accumulate=accumulate_dq, ds=buf)  # fmt: skip
+                         accumulate=accumulate_dq, ds=buf, dq_final=None if dq_final is None else dq_final[:, :, q_h],
+                         dq_final_rows=dq_final_rows)  # fmt: skip
     return buf.numel()
 
 
 def attn_bwd_dkdv_into(
     q, k, v, dout, lse, delta, dk: torch.Tensor, dv: torch.Tensor, softmax_scale: float, causal: bool,
     accumulate: bool = False, k_pe: torch.Tensor = None, dk_pe: torch.Tensor = None, ds: torch.Tensor = None,
+    zero_tail: int = 0,
 ) -> None:  # fmt: skip
     """dk, dv <- (or +=, with accumulate) the gradients of this chunk pair; bf16 or fp32 outputs.
+    zero_tail: dk and dv are row ranges [:skv] of tensors with at least skv + zero_tail rows, and the kernel
+    also clears those rows behind them (not with accumulate, not dk_pe).
     With k_pe (see attn_fwd_into) dk is the gradient of k_nope and dk_pe [b, skv, 64] (contiguous rows,
     same dtype as dk) receives the gradient of k_pe, summed over heads in head order.
     ds: uint8 buffer of attn_bwd_ds_bytes(q, k, v, causal) bytes; the kernel leaves its dS tiles there for an
@@ -316,6 +322,7 @@ def attn_bwd_dkdv_into(
     assert dk_rh == dv_rh == args.kv_row_heads, "dk / dv must be laid out like k / v"
     args.dkv_dtype = _C.dtype_code(dk)
     args.accumulate_dkv = int(bool(accumulate))
+    args.dkv_zero_tail = int(zero_tail)
     # Scratch for the head-split partial sums; the caching allocator makes this a pointer bump,
     # and stream ordering keeps the block alive until the kernels that use it have run.
     need = _C.lib().pith_attn_bwd_dkdv_workspace_bytes(_C.byref(args))
@@ -328,9 +335,12 @@ def attn_bwd_dkdv_into(
 
 def attn_bwd_dq_into(
     q, k, v, dout, lse, delta, dq: torch.Tensor, softmax_scale: float, causal: bool, accumulate: bool = False,
-    k_pe: torch.Tensor = None, ds: torch.Tensor = None,
+    k_pe: torch.Tensor = None, ds: torch.Tensor = None, dq_final: torch.Tensor = None, dq_final_rows=None,
 ) -> None:  # fmt: skip
     """dq <- (or +=, with accumulate) the query gradient of this chunk pair; bf16 or fp32 output.
+    dq_final (bf16, laid out like an fp32 dq; head dims in FINAL_DQ_HEAD_DIMS): rows dq_final_rows ((begin, end)
+    on multiples of 32, None = all) receive their complete value, what dq held included when accumulating,
+    rounded to bf16 in dq_final instead of dq.
     ds: the buffer an attn_bwd_dkdv_into call on the same chunk pair has just filled; dq is then
     computed from those dS tiles without recomputing the scores."""
     args = _bwd_args(q, k, v, dout, lse, delta, softmax_scale, causal, k_pe)
@@ -342,6 +352,14 @@ def attn_bwd_dq_into(
     assert dq_rh == args.q_row_heads, "dq must be laid out like q"
     args.dq_dtype = _C.dtype_code(dq)
     args.accumulate_dq = int(bool(accumulate))
+    if dq_final is not None:
+        _C.require_device(q, dq_final)
+        assert dq_final.dtype == torch.bfloat16 and dq_final.shape == q.shape, "dq_final must be a bf16 tensor shaped like q"
+        args.dq_final_bs, fin_rh = _C.bshd_head_range_strides(dq_final, "dq_final")
+        assert fin_rh == args.q_row_heads, "dq_final must be laid out like q"
+        args.dq_final = dq_final.data_ptr()
+        if dq_final_rows is not None:
+            args.dq_final_rows[0], args.dq_final_rows[1] = dq_final_rows
     _C.check(_C.lib().pith_attn_bwd_dq(_C.byref(args), _C.current_stream(q)))
 
 

@@ -42,6 +42,7 @@ import torch
 
 from pithtrain_amd import _C
 from pithtrain_amd.operators.mla.hip import (
+    FINAL_DQ_HEAD_DIMS,
     MERGING_HEAD_DIMS,
     attn_bwd_delta_into,
     attn_bwd_pair_into,
@@ -53,6 +54,12 @@ LAYOUTS = ("contiguous", "zigzag")
 # Ring steps after the first merge inside the forward kernel (one launch per step) where the kernels support it;
 # False restores chunk forward + combine launch per step (kept for comparison runs).
 FUSE_MERGE = True
+# The ring backward lets the dQ launch that completes a row range write its bf16 rows (no cast pass at the end)
+# where the kernels support it; False restores the fp32 accumulator + cast (kept for comparison runs).
+FUSE_FINAL_DQ = True
+# The dK/dV launch of a step that sees only the first rows of a chunk clears the other rows of dk / dv itself;
+# False restores separate fill launches.
+FUSE_ZERO_TAIL = True
 
 
 @dataclass(frozen=True)
@@ -253,6 +260,15 @@ class RingBackward:
         self.dout = dout.contiguous()
         self.q, self.lse, self.scale, self.steps = q, lse, softmax_scale, list(steps)
         B, S, H, _ = q.shape
+        # Rows between two boundaries of the steps' query ranges receive the same contributions; `dq_left` counts
+        # those still to come. Where the kernels can, the step that brings a range's last contribution writes its
+        # bf16 rows of dq itself (and leaves them out of the fp32 accumulator); ranges finished that way need no
+        # cast at the end.
+        cuts = sorted({0, S} | {r for st in self.steps for r in st.q_rows})
+        self.dq_ranges = list(zip(cuts[:-1], cuts[1:]))
+        self.dq_left = {r: sum(st.q_rows[0] <= r[0] and r[1] <= st.q_rows[1] for st in self.steps) for r in self.dq_ranges}
+        self.dq_done_in_kernel = set()
+        self.final_in_kernel = FUSE_FINAL_DQ and (q.shape[-1], out.shape[-1]) in FINAL_DQ_HEAD_DIMS and len(self.steps) > 1
         # delta from the COMBINED output, once (pithtrain/operators/ring_attention/mla.py:101).
         self.delta = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
         attn_bwd_delta_into(out, self.dout, self.delta)
@@ -274,6 +290,7 @@ class RingBackward:
         if k_pe_j is not None and k_pe_j.dim() == 4:
             k_pe_j = k_pe_j[:, :, 0]
         dk_pe_j = None
+        zero_tail = 0
         if add_to is None:
             dk_j, dv_j = torch.empty_like(k_j), torch.empty_like(v_j)
             outs = [dk_j, dv_j]
@@ -281,7 +298,10 @@ class RingBackward:
                 dk_pe_j = torch.empty((k_j.shape[0], k_j.shape[1], k_pe_j.shape[-1]), dtype=k_j.dtype, device=k_j.device)
                 outs.append(dk_pe_j)
             if st.kv_rows != (0, k_j.shape[1]):  # rows of the chunk this rank cannot see get no gradient
-                for t in outs:
+                # rows behind the visible ones are cleared by the dK/dV launch itself; anything else here
+                in_kernel = FUSE_ZERO_TAIL and st.kv_rows[0] == 0
+                zero_tail = k_j.shape[1] - st.kv_rows[1] if in_kernel else 0
+                for t in outs if not in_kernel else outs[2:]:  # (the launch does not clear dk_pe)
                     t[:, : st.kv_rows[0]].zero_()
                     t[:, st.kv_rows[1] :].zero_()
         else:
@@ -295,17 +315,37 @@ class RingBackward:
         # dK/dV, then dQ; the pair helper decides whether the dK/dV kernel leaves its dS tiles for the dQ
         # kernel (head dims 128/128, bounded scratch) or both kernels recompute the scores.
         # Step 0 covers every row and initialises the dQ accumulator; later steps add to their rows.
+        covered = [r for r in self.dq_ranges if st.q_rows[0] <= r[0] and r[1] <= st.q_rows[1]]
+        for r in covered:
+            self.dq_left[r] -= 1
+        final = final_rows = None
+        if self.final_in_kernel:
+            last = [r for r in covered if self.dq_left[r] == 0]
+            span = (last[0][0] - st.q_rows[0], last[-1][1] - st.q_rows[0]) if last else None
+            n_q = st.q_rows[1] - st.q_rows[0]
+            if last and sum(r[1] - r[0] for r in last) == span[1] - span[0] and span[0] % 32 == 0 and (
+                span[1] % 32 == 0 or span[1] == n_q
+            ):
+                final, final_rows = _rows(self.dq, st.q_rows), span
+                self.dq_done_in_kernel.update(last)
         self.scratch_bytes = max(self.scratch_bytes, attn_bwd_pair_into(
             qs, ks, vs, ds, ls, dl, _rows(self.dq_acc, st.q_rows), _rows(dk_j, st.kv_rows), _rows(dv_j, st.kv_rows),
             self.scale, st.causal, accumulate_dq=self.done > 0, accumulate_dkv=add_to is not None, k_pe=pes,
-            dk_pe=_pe_rows(dk_pe_j, st.kv_rows), handover=self.handover))  # fmt: skip
+            dk_pe=_pe_rows(dk_pe_j, st.kv_rows), handover=self.handover, zero_tail=zero_tail,
+            dq_final=final, dq_final_rows=final_rows))  # fmt: skip
         self.done += 1
         return (dk_j, dv_j) if k_pe_j is None else (dk_j, dv_j, dk_pe_j)
 
     def finish(self) -> torch.Tensor:
         assert self.done == len(self.steps), "not every ring step has run"
         if self.dq_acc is not self.dq:
-            cast_f32_bf16_into(self.dq_acc, self.dq)
+            todo = [r for r in self.dq_ranges if r not in self.dq_done_in_kernel]
+            if len(todo) == len(self.dq_ranges):
+                cast_f32_bf16_into(self.dq_acc, self.dq)
+            else:
+                for r in todo:  # ranges no launch could finish (boundaries off the 32-row grid)
+                    for b in range(self.dq.shape[0]):
+                        cast_f32_bf16_into(self.dq_acc[b, r[0] : r[1]], self.dq[b, r[0] : r[1]])
         return self.dq
 
 

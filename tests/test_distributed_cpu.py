@@ -48,10 +48,14 @@ def _install_cpu_stand_ins():
         dq.copy_(dq.double() + rdq if accumulate else rdq)
 
     def attn_bwd_pair_into(q, k, v, dout, lse, delta, dq, dk, dv, scale, causal, accumulate_dq=False,
-                           accumulate_dkv=False, k_pe=None, dk_pe=None, handover=True):  # fmt: skip
+                           accumulate_dkv=False, k_pe=None, dk_pe=None, handover=True, zero_tail=0, dq_final=None,
+                           dq_final_rows=None):  # fmt: skip
+        assert zero_tail == 0 and dq_final is None, "the stand-ins do not implement the fused conveniences"
         attn_bwd_dkdv_into(q, k, v, dout, lse, delta, dk, dv, scale, causal, accumulate_dkv, k_pe, dk_pe)
         attn_bwd_dq_into(q, k, v, dout, lse, delta, dq, scale, causal, accumulate_dq, k_pe)
         return 0  # no dS hand-over between the stand-ins
+
+    L.FUSE_FINAL_DQ = L.FUSE_ZERO_TAIL = False  # per-process (the ranks are spawned): fill and cast stay separate calls
 
     def combine_into(out1, lse1, out2, lse2, out, lse_out, base=0):
         o, l = R.combine_log2(out1.double(), lse1.double(), out2.double(), lse2.double())

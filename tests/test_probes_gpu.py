@@ -1,0 +1,56 @@
+"""Runs the two device probes of tests/probes/ (built ahead of time by __graft_entry__.build()) and checks what the
+design argues from: the full-chip rate of bf16 matrix instructions depends on the operand data and stays below the
+nominal peak with random operands, and fp32 global atomic adds are far too slow to accumulate dQ in a single backward
+kernel. The probes print their tables; profiles/ holds a copy with hardware counters beside it."""
+
+import os
+import re
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "probes", "bin")
+
+
+def _run(name):
+    path = os.path.join(BIN, name)
+    if not os.path.exists(path):
+        pytest.fail(f"{path} is missing: build it with `python tests/probes/build_probes.py`")
+    proc = subprocess.run([path], capture_output=True, text=True, timeout=150)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    print(proc.stdout)
+    return proc.stdout.splitlines()
+
+
+def test_matrix_rate_depends_on_operand_data(gpu):
+    rows = {}
+    for line in _run("mfma_rate_probe"):
+        m = re.match(r"(.+?)\s+fragments (\d+) blocks (\d+):\s+([\d.]+) ms\s+(\d+) TFLOP/s", line)
+        if m:
+            rows[(m.group(1).strip(), int(m.group(2)), int(m.group(3)))] = float(m.group(5))
+    assert len(rows) == 18, rows
+    const = [v for (name, _, _), v in rows.items() if name.startswith("constants")]
+    rand = [v for (name, _, _), v in rows.items() if name.startswith("random")]
+    assert all(500 < v < 2600 for v in const + rand), rows  # nominal dense bf16 peak: 2500 TFLOP/s
+    # constants toggle no operand bits and get close to the nominal peak; random operands stay well below it, in
+    # every launch shape (single rows vary with the power state the launch finds: the best of each kind is compared)
+    assert max(const) > 0.9 * 2500, rows
+    assert max(rand) < 0.8 * 2500 and max(const) > 1.15 * max(rand), rows
+
+
+def test_fp32_atomic_rate_is_far_below_what_a_fused_backward_needs(gpu):
+    rows = {}
+    for line in _run("atomic_rate_probe"):
+        m = re.match(r"(.+?)\s+grid\s+(\d+)\s+([\d.]+) ms\s+atomic\s+([\d.]+) GB/s\s+wrong elements (\d+)", line)
+        if m:
+            rows[m.group(1).strip()] = (float(m.group(3)), float(m.group(4)), int(m.group(5)))
+    assert len(rows) == 8, rows
+    assert all(wrong == 0 for _, _, wrong in rows.values()), rows  # the sums are right in every variant
+    rates = [gbps for name, (_, gbps, _) in rows.items() if "atomics" in name]
+    # a fused kernel would have to add 4.3 GB per launch inside the 0.45 ms of recomputation it saves: 9.5 TB/s
+    assert max(rates) < 4000, rows
+    # atomics and the matrix load overlap: together they take about as long as the slower of the two
+    alone, both = rows["atomics only, device scope, dkdv mapping"][0], rows["mfma 40 + atomics, device scope"][0]
+    assert both < 1.25 * max(alone, rows["mfma only (40 per wave-interval)"][0]), rows

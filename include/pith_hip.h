@@ -203,7 +203,7 @@ int pith_attn_bwd_delta(const pith_attn_delta_args* args, pith_stream_t stream);
  *   dkv_zero_tail: pith_attn_bwd_dkdv also sets rows [Skv, Skv + dkv_zero_tail) of dk and dv to
  *     zero (not dk_pe; ignored with accumulate_dkv): the rows of a chunk that a zigzag step does not
  *     see owe a zero gradient.
- *   dq_final (pith_attn_bwd_dq, dq_dtype PITH_F32, head dims (128,128)): query rows
+ *   dq_final (pith_attn_bwd_dq, dq_dtype PITH_F32, head dims (128,128) or (192,128)): query rows
  *     [dq_final_rows[0], dq_final_rows[1]) (multiples of 32 or Sq; {0,0} = all) receive their
  *     result - the old contents of dq included when accumulate_dq is set - rounded to bf16 in
  *     dq_final [B,Sq,Hq,Dqk] (laid out like dq) instead of dq: the last ring step that touches a row

@@ -328,8 +328,8 @@ extern "C" int pith_attn_bwd_dq(const pith_attn_bwd_args* a, pith_stream_t strea
   if (rc != PITH_OK) return rc;
   BwdParams p = make_bwd_params(a);
   if (a->dq_final) {
-    if (a->dq_dtype != PITH_F32 || a->Dqk != 128 || a->Dv != 128)
-      return fail(PITH_ERR_UNSUPPORTED, "pith_attn_bwd_dq: dq_final needs an fp32 dq and head dims (128,128)");
+    if (a->dq_dtype != PITH_F32 || a->Dv != 128 || (a->Dqk != 128 && a->Dqk != 192))
+      return fail(PITH_ERR_UNSUPPORTED, "pith_attn_bwd_dq: dq_final needs an fp32 dq and head dims (128,128) or (192,128)");
     if (!aligned16(a->dq_final) || a->dq_final_bs % 8)
       return fail(PITH_ERR_MISALIGNED, "pith_attn_bwd_dq: dq_final pointer / batch stride must keep 16-byte alignment");
     int64_t r0 = a->dq_final_rows[0], r1 = a->dq_final_rows[1];

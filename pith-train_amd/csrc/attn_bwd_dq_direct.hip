@@ -440,13 +440,24 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
     store_rows32_via_lds<OutT, DB>(exch, dqh + q_wave0 * q_row_stride, q_row_stride, p.Sq - q_wave0, acc, p.scale, p.accumulate != 0, lane, fin);
   } else if (qrow < p.Sq) {
     OutT* dst = dqh + qrow * q_row_stride;
+    // rows whose gradient is complete with this call go out as bf16 (an fp32 dq only; the same for the whole wave)
+    const bool fin = sizeof(OutT) == 4 && p.dq_final != nullptr && q_wave0 >= p.final_r0 && q_wave0 < p.final_r1;
+    __bf16* fdst = p.dq_final + b * p.dq_final_bs + (int64_t)h * DQK + qrow * q_row_stride;
 #pragma unroll
     for (int o = 0; o < DB; ++o)
 #pragma unroll
       for (int b4 = 0; b4 < 4; ++b4) {
         const f32x4 v4 = *reinterpret_cast<const f32x4*>(exch + ((o * 4 + b4) * 64 + lane) * 16);
-        store4<OutT>(dst + 32 * o + 8 * b4 + 4 * g, (acc[o][4 * b4] + v4[0]) * p.scale, (acc[o][4 * b4 + 1] + v4[1]) * p.scale,
-                     (acc[o][4 * b4 + 2] + v4[2]) * p.scale, (acc[o][4 * b4 + 3] + v4[3]) * p.scale, p.accumulate != 0);
+        const int col = 32 * o + 8 * b4 + 4 * g;
+        if (fin) {
+          f32x4 x = {(acc[o][4 * b4] + v4[0]) * p.scale, (acc[o][4 * b4 + 1] + v4[1]) * p.scale,
+                     (acc[o][4 * b4 + 2] + v4[2]) * p.scale, (acc[o][4 * b4 + 3] + v4[3]) * p.scale};
+          if (p.accumulate) x += *reinterpret_cast<const f32x4*>(dst + col);
+          store4<__bf16>(fdst + col, x[0], x[1], x[2], x[3], false);
+        } else {
+          store4<OutT>(dst + col, (acc[o][4 * b4] + v4[0]) * p.scale, (acc[o][4 * b4 + 1] + v4[1]) * p.scale,
+                       (acc[o][4 * b4 + 2] + v4[2]) * p.scale, (acc[o][4 * b4 + 3] + v4[3]) * p.scale, p.accumulate != 0);
+        }
       }
   }
 }

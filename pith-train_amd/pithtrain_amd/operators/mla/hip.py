@@ -68,7 +68,7 @@ def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool, 
 
 
 MERGING_HEAD_DIMS = ((128, 128), (192, 128))  # forward kernels that can merge with a running result
-FINAL_DQ_HEAD_DIMS = ((128, 128),)  # dQ kernels that can emit finished rows as bf16 beside an fp32 accumulator
+FINAL_DQ_HEAD_DIMS = ((128, 128), (192, 128))  # dQ kernels that can emit finished rows as bf16 beside an fp32 accumulator
 
 
 def attn_fwd_into(

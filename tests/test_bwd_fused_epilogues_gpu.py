@@ -49,20 +49,22 @@ def test_dkdv_clears_the_rows_behind_the_visible_part(gpu, Dqk, Hq, Hkv, dtype):
     assert (dk2[:, Skv:] == 1).all() and (dv2[:, Skv:] == 1).all()
 
 
-# (Sq, Skv, Hq, Hkv, hand-over): the three dQ kernels for head dims (128, 128)
+# (Sq, Skv, Hq, Hkv, hand-over, Dqk): the three dQ kernels for head dims (128, 128) and the one for (192, 128)
 DQ_KERNELS = [
-    pytest.param(2048, 1024, 32, 4, True, id="from-dS-images"),
-    pytest.param(2048, 1024, 32, 4, False, id="recomputing-256-row"),
-    pytest.param(640, 320, 4, 2, False, id="recomputing-128-row"),
-    pytest.param(1000, 520, 8, 2, False, id="ragged"),
+    pytest.param(2048, 1024, 32, 4, True, 128, id="from-dS-images"),
+    pytest.param(2048, 1024, 32, 4, False, 128, id="recomputing-256-row"),
+    pytest.param(640, 320, 4, 2, False, 128, id="recomputing-128-row"),
+    pytest.param(1000, 520, 8, 2, False, 128, id="ragged"),
+    pytest.param(1024, 512, 16, 16, False, 192, id="mla-192"),
+    pytest.param(333, 200, 4, 4, False, 192, id="mla-192-ragged"),
 ]
 
 
-@pytest.mark.parametrize("Sq,Skv,Hq,Hkv,handover", DQ_KERNELS)
+@pytest.mark.parametrize("Sq,Skv,Hq,Hkv,handover,Dqk", DQ_KERNELS)
 @pytest.mark.parametrize("accumulate", [True, False])
-def test_dq_final_rows_equal_accumulate_then_cast(gpu, Sq, Skv, Hq, Hkv, handover, accumulate):
+def test_dq_final_rows_equal_accumulate_then_cast(gpu, Sq, Skv, Hq, Hkv, handover, Dqk, accumulate):
     B = 1
-    q, k, v, dout, scale = _inputs(B, Sq, Skv, Hq, Hkv, 128, seed=5)
+    q, k, v, dout, scale = _inputs(B, Sq, Skv, Hq, Hkv, Dqk, seed=5)
     qd, kd, vd, dod = (t.to(gpu) for t in (q, k, v, dout))
     o, lse = H._mla_fwd(qd, kd, vd, scale, False)
     delta = H._mla_bwd_preprocess(o, dod)
@@ -89,14 +91,14 @@ def test_dq_final_rows_equal_accumulate_then_cast(gpu, Sq, Skv, Hq, Hkv, handove
 
 
 @pytest.mark.parametrize("layout", ["contiguous", "zigzag"])
-@pytest.mark.parametrize("Hq,Hkv,S", [(8, 2, 2048), (32, 4, 4096), (4, 4, 1000)])
-def test_ring_backward_with_and_without_the_fused_epilogues(gpu, layout, Hq, Hkv, S, monkeypatch):
+@pytest.mark.parametrize("Hq,Hkv,S,D", [(8, 2, 2048, 128), (32, 4, 4096, 128), (4, 4, 1000, 128), (4, 4, 2048, 192)])
+def test_ring_backward_with_and_without_the_fused_epilogues(gpu, layout, Hq, Hkv, S, D, monkeypatch):
     """Every rank of a ring of 4: dQ, dK, dV bit for bit the same whether the fill and the cast are separate
     launches or folded into the dK/dV and dQ launches, and equal to the oracle's ring share."""
-    B, C, D = 1, 4, 128
+    B, C = 1, 4
     g = torch.Generator().manual_seed(13)
     scale = D**-0.5
-    full = [torch.randn(B, S, h, D, generator=g).to(torch.bfloat16) for h in (Hq, Hkv, Hkv, Hq)]
+    full = [torch.randn(B, S, h, d, generator=g).to(torch.bfloat16) for h, d in ((Hq, D), (Hkv, D), (Hkv, 128), (Hq, 128))]
     split = (lambda x: R.zigzag_split(x, C)) if layout == "zigzag" else (lambda x: [c.contiguous() for c in x.chunk(C, 1)])
     if layout == "zigzag" and S % (2 * C):
         pytest.skip("zigzag needs 2 * cp_size blocks")

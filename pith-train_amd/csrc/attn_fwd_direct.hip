@@ -56,7 +56,13 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   constexpr bool kSumTest = !(DQK == 192 && !HALF);  // how the softmax decides to refresh its running maximum
   // the tile rings; the epilogue reuses them to turn the output tile (one area per storing wave)
   constexpr int kRings = kSlots * (kKTile + kTile), kTurn = (HALF ? kWaves / 2 : kWaves) * kRowsViaLdsBytes<DVB>;
-  __shared__ __attribute__((aligned(1024))) char smem[kRings > kTurn ? kRings : kTurn];
+  // 256-row workgroups for 128 features fetch their query block through LDS as well (four 64-row tiles into the three
+  // ring slots that are still empty while the first tiles land, and one more tile behind the rings): whole-row direct
+  // loads instead of 32-byte pieces of 32 different rows per instruction
+  constexpr bool kQViaLds = DQK == 128 && !HALF;
+  constexpr int kQSpill = kRings;  // where the fourth query tile goes
+  constexpr int kNeed = kQViaLds ? kRings + kTile : kRings;
+  __shared__ __attribute__((aligned(1024))) char smem[kNeed > kTurn ? kNeed : kTurn];
   char* const kbuf = smem;
   char* const vbuf = smem + kSlots * kKTile;
 
@@ -123,7 +129,22 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
 
   // Q^T fragments (B operand): column = query row, slots = 8 consecutive features.
   bf16x8 qf[KS];
-  {
+  // LDS homes of the workgroup's four 64-row query tiles (kQViaLds): K slot 3, V slots 2 and 3, behind the rings
+  auto q_home = [&](int t) __attribute__((always_inline)) -> char* {
+    return t == 0 ? kbuf + 3 * kKTile : t == 1 ? vbuf + 2 * kTile : t == 2 ? vbuf + 3 * kTile : smem + kQSpill;
+  };
+  if constexpr (kQViaLds) {
+    DirectTile128<kBN, kThreads> qmover;
+    qmover.init((int)(q_row_stride * 2), wave, lane);
+    const char* qsrc = reinterpret_cast<const char*>(qh);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      // rows beyond Sq repeat the last row (their results are never stored); a tile wholly beyond Sq is skipped by
+      // clamping its first row, which keeps the number of load instructions per wave fixed
+      const int row0 = min(m0 + t * kBN, p.Sq - 1);
+      qmover.issue(qsrc + (int64_t)row0 * q_row_stride * 2, p.Sq - row0, q_home(t), wave, lane);
+    }
+  } else {
     const int row = qrow < p.Sq ? qrow : p.Sq - 1;
     const __bf16* src = qh + row * q_row_stride + g * 8;
 #pragma unroll
@@ -337,6 +358,12 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   // ---- prologue: S(0) (and P(0) in the early waves) from K tile 0
   __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far, Q fragments included
   __syncthreads();
+  if constexpr (kQViaLds) {
+    // this wave's 32 rows: tile wave / 2, row block wave % 2 (the slots are refilled only after the next barrier)
+    const char* qt = q_home(wave >> 1) + (wave & 1) * 32 * kRowBytes128;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qt + straight_offset128(c, 2 * ks + g));
+  }
   scores(kbuf);
   __syncthreads();  // K tile 0 has been read by every wave: its slot may be refilled
   if (!late) softmax(0);

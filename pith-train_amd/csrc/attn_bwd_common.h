@@ -47,6 +47,8 @@ struct BwdParams {
   int final_r0, final_r1;
   // dK/dV kernels: blocks main_blocks .. of the grid clear rows [Skv, Skv + zero_tail) of dk and dv
   int zero_tail, main_blocks;
+  // dK/dV for head dims (128, 128), causal: launch the instance that visits the query tiles from the last one down
+  int walk_desc;
 };
 
 constexpr int kZeroTailRows = 32;  // rows one such block clears
@@ -155,6 +157,25 @@ __device__ __forceinline__ void store_rows32(OutT* block, int64_t row_stride, in
         }
       }
     }
+  }
+}
+
+// dK/dV kernels: linear block id -> (key tile, position within a level), a level being the `per_level` (kv head,
+// batch, head part) combinations of one key tile; early key tiles first: under the causal mask they see the most
+// query tiles. Each combination streams its own Q / dO tiles. With more than 8 of them and at least kChunkedTiles
+// key tiles they are taken in chunks of 8, all key tiles of a chunk before the next chunk, so that the workgroups
+// one XCD holds at a time (block id mod 8) belong to one combination and share its Q / dO stream through that
+// XCD's L2 (see decode_block for the measurements behind the threshold).
+__device__ __forceinline__ void decode_dkdv_block(int linear, int per_level, int tiles, int& n_tile, int& pos) {
+  if (tiles >= kChunkedTiles && per_level > 8 && (per_level & 7) == 0) {
+    const int per_chunk = 8 * tiles;
+    const int c = linear / per_chunk;
+    const int rem = linear - c * per_chunk;
+    n_tile = rem >> 3;
+    pos = c * 8 + (rem & 7);
+  } else {
+    n_tile = linear / per_level;
+    pos = linear - n_tile * per_level;
   }
 }
 

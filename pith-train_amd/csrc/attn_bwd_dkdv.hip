@@ -160,11 +160,10 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(BwdParams p) {
   const int pair = wave & 3;
   const bool role_b = wave >= 4;
 
-  // linear block id -> (key tile, kv head, batch, head part); early key tiles first: under the
-  // causal mask they see the most query tiles
+  // linear block id -> (key tile, kv head, batch, head part)
   const int per_level = p.Hkv * p.B * p.split;
-  const int n_tile = blockIdx.x / per_level;
-  int pos = blockIdx.x - n_tile * per_level;
+  int n_tile, pos;
+  decode_dkdv_block(blockIdx.x, per_level, p.tiles, n_tile, pos);
   const int part = pos % p.split;
   pos /= p.split;
   const int hk = pos % p.Hkv, b = pos / p.Hkv;
@@ -327,6 +326,8 @@ int64_t dkpe_bytes_for(const pith_attn_bwd_args* a) {
 }
 int64_t workspace_bytes_for(const pith_attn_bwd_args* a, int split) { return split_bytes_for(a, split) + dkpe_bytes_for(a); }
 
+constexpr int64_t kWalkDescBytes = 192ll << 20;
+
 template <int DQK, int DV>
 void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
   p.tiles = (int)((a->Skv + kBN - 1) / kBN);
@@ -336,6 +337,8 @@ void launch_dkdv(BwdParams p, const pith_attn_bwd_args* a, hipStream_t st) {
   const dim3 grid((unsigned)(p.main_blocks + (p.zero_tail + kZeroTailRows - 1) / kZeroTailRows)), block(kThreads);
   const bool f32 = a->dkv_dtype == PITH_F32;
   if constexpr (DQK == 128 && DV == 128) {
+    // descending walk under the mask when Q and dO together exceed what the last-level cache (256 MB) keeps
+    p.walk_desc = a->causal != 0 && (int64_t)a->B * a->Sq * a->Hq * (DQK + DV) * 2 > kWalkDescBytes;
     launch_dkdv_d128(p, a->causal != 0, f32, grid.x, st);
   } else if constexpr (DQK == 192 && DV == 128) {
     launch_dkdv_d192(p, a->causal != 0, f32, grid.x, st);

@@ -43,11 +43,27 @@ constexpr int kSmem = kStages * kStage + 4 * kExchPair;
 constexpr int kDsStoresPerInterval = kBM / 16;
 static_assert(kDsStoresPerInterval == 4, "make_ds stores frag[0..3]; the vmcnt immediate below has a 4-bit low field");
 
-// Position of a query tile in the stream of (query head, tile) pairs a workgroup visits.
+// Position of a query tile in the stream of (query head, tile) pairs a workgroup visits, and the order of that
+// stream. Ascending: head by head, tiles upwards. Descending (DESC): tiles from the last one down with the heads
+// innermost. Under the mask a workgroup starts at its diagonal, so in ascending order the workgroups of an XCD stand
+// on different tiles of the Q / dO stream they share and each fetches it from beyond L2 again; descending, all of
+// them start on the last tile together. Measured: the causal launch over 16384 rows x 64 heads (34 GB fetched per launch, Q and dO
+// are 537 MB) 5-7 % faster; over 8192 rows x 32 heads (134 MB, which the 256 MB last-level cache holds) 0-2 %
+// slower; non-causal launches, whose workgroups walk in step either way, 1-3 % slower. The host picks by size
+// (BwdParams::walk_desc selects the DESC instances of the causal kernel).
+template <bool DESC>
 struct TileCursor {
   int hq, mt;
-  __device__ __forceinline__ void advance(int m_first, int m_end) {
-    if (++mt == m_end) {
+  __device__ __forceinline__ static TileCursor first(int hq0, int m_first, int m_end) {
+    return TileCursor{hq0, DESC ? m_end - 1 : m_first};
+  }
+  __device__ __forceinline__ void advance(int m_first, int m_end, int hq0, int hq_end) {
+    if (DESC) {
+      if (++hq == hq_end) {
+        hq = hq0;
+        --mt;
+      }
+    } else if (++mt == m_end) {
       mt = m_first;
       ++hq;
     }
@@ -61,7 +77,7 @@ struct TileCursor {
 // 1 KB per 16-row step j, the 16 bytes of lane (g, c) at g*512 + ((c ^ 8g ^ 4(j&1)) << 4) (the
 // XOR terms make the reader's transposing LDS reads conflict-free). Keys at or beyond Skv hold 0
 // (their P is masked to 0).
-template <bool CAUSAL, typename OutT, bool EMIT_DS>
+template <bool CAUSAL, typename OutT, bool EMIT_DS, bool DESC = false>
 __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams p) {
   constexpr int KS = kD / 16, DB = kD / 32;
   __shared__ __attribute__((aligned(1024))) char smem[kSmem];
@@ -76,11 +92,10 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   const int pair = wave & 3;
   const bool role_b = wave >= 4;
 
-  // linear block id -> (key tile, kv head, batch, head part); early key tiles first: under the
-  // causal mask they see the most query tiles
+  // linear block id -> (key tile, kv head, batch, head part)
   const int per_level = p.Hkv * p.B * p.split;
-  const int n_tile = blockIdx.x / per_level;
-  int pos = blockIdx.x - n_tile * per_level;
+  int n_tile, pos;
+  decode_dkdv_block(blockIdx.x, per_level, p.tiles, n_tile, pos);
   const int part = pos % p.split;
   pos /= p.split;
   const int hk = pos % p.Hkv, b = pos / p.Hkv;
@@ -105,7 +120,9 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   mover.init(q_row_bytes, pair, lane);
   const char* q_base = reinterpret_cast<const char*>(p.q + b * p.q_bs);
   const char* do_base = reinterpret_cast<const char*>(p.dout + b * p.dout_bs);
-  TileCursor req = {hq0, m_first};
+  using Cursor = TileCursor<DESC>;
+  const int hq_end = hq0 + heads_per_part;
+  Cursor req = Cursor::first(hq0, m_first, m_end);
   auto request = [&](char* stage) __attribute__((always_inline)) {
     const int row0 = req.mt * kBM;
     const int64_t head_off = (int64_t)req.hq * kD * 2 + (int64_t)row0 * q_row_bytes;
@@ -117,7 +134,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
       const float* src = (pair == 0 ? p.lse : p.delta) + b * p.lse_bs + (int64_t)req.hq * p.lse_hs + row;
       load_lds4(src, stage + 2 * kTile + pair * kBM * 4);
     }
-    req.advance(m_first, m_end);
+    req.advance(m_first, m_end, hq0, hq_end);
   };
   if (n_iter > 0 && role_b) request(smem);
 
@@ -295,7 +312,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   // writes per interval in flight next to 33 KB of tile reads, its vector cache stalls on pending
   // requests three times as often, and the sustained clock drops by 6 % under the write traffic.
   char* const ds_wg = EMIT_DS ? p.ds + ((int64_t)n_tile * 4 + pair) * 4096 : nullptr;
-  auto make_ds = [&](const char* stage, const TileCursor& tile) __attribute__((always_inline)) {
+  auto make_ds = [&](const char* stage, const Cursor& tile) __attribute__((always_inline)) {
     f32x4 pr[2][4];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
@@ -330,7 +347,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
   // Ring stages rotate: prev <- cur <- next <- (the stage prev used to be).
   auto run = [&](auto role_tag) __attribute__((always_inline)) {
     constexpr bool ROLE_B = decltype(role_tag)::value;
-    TileCursor cur = {hq0, m_first}, done = cur;  // tiles i and i-1 of interval i
+    Cursor cur = Cursor::first(hq0, m_first, m_end), done = cur;  // tiles i and i-1 of interval i
     int off_prev = 2 * kStage, off_cur = 0, off_next = kStage;
     auto end_interval = [&](bool stored) __attribute__((always_inline)) {
       // the tile requested in this interval has landed. Vector memory operations complete in issue
@@ -340,7 +357,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d128_kernel(BwdParams 
       else __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
       done = cur;
-      cur.advance(m_first, m_end);
+      cur.advance(m_first, m_end, hq0, hq_end);
       const int t = off_prev;
       off_prev = off_cur;
       off_cur = off_next;
@@ -425,7 +442,10 @@ template <bool EMIT_DS>
 static void launch_variant(const BwdParams& p, bool causal, bool f32_out, unsigned grid, hipStream_t st) {
   const dim3 g(grid), block(kThreads);
   if (causal) {
-    if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, float, EMIT_DS>), g, block, 0, st, p);
+    if (p.walk_desc) {
+      if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, float, EMIT_DS, true>), g, block, 0, st, p);
+      else hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, __bf16, EMIT_DS, true>), g, block, 0, st, p);
+    } else if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, float, EMIT_DS>), g, block, 0, st, p);
     else hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<true, __bf16, EMIT_DS>), g, block, 0, st, p);
   } else {
     if (f32_out) hipLaunchKernelGGL((attn_bwd_dkdv_d128_kernel<false, float, EMIT_DS>), g, block, 0, st, p);

@@ -101,11 +101,10 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_d192_kernel(BwdParams 
   const int pair = wave & 3;
   const bool role_b = wave >= 4;
 
-  // linear block id -> (key tile, kv head, batch, head part); early key tiles first: under the
-  // causal mask they see the most query tiles
+  // linear block id -> (key tile, kv head, batch, head part)
   const int per_level = p.Hkv * p.B * p.split;
-  const int n_tile = blockIdx.x / per_level;
-  int pos = blockIdx.x - n_tile * per_level;
+  int n_tile, pos;
+  decode_dkdv_block(blockIdx.x, per_level, p.tiles, n_tile, pos);
   const int part = pos % p.split;
   pos /= p.split;
   const int hk = pos % p.Hkv, b = pos / p.Hkv;

@@ -32,7 +32,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_bwd_dq_kernel(BwdParams p) {
   const int lane = tid & 63, wave = tid >> 6;
   const int c = lane & 31, g = lane >> 5;
   int m_tile, h, b;
-  decode_block(blockIdx.x, p.Hq, p.B, p.tiles, m_tile, h, b);
+  decode_block(blockIdx.x, p.Hq, p.B, p.tiles, p.group, m_tile, h, b);
   const int hk = h / p.group;
   const int m0 = m_tile * BM;
   const int q_wave0 = m0 + wave * ROWS_WAVE;
@@ -305,7 +305,7 @@ BwdParams make_bwd_params(const pith_attn_bwd_args* a) {
   p.ds_kb = (int)((a->Skv + kDkdvBlockN - 1) / kDkdvBlockN);
   p.ds_hs = (a->causal ? ds_tile_start<true>(p.ds_qt, p.ds_kb) : ds_tile_start<false>(p.ds_qt, p.ds_kb)) * kDsBlockBytes;
   p.dq_final = nullptr; p.dq_final_bs = 0; p.final_r0 = p.final_r1 = 0;
-  p.zero_tail = 0; p.main_blocks = 0x7fffffff;
+  p.zero_tail = 0; p.main_blocks = 0x7fffffff; p.walk_desc = 0;
   return p;
 }
 

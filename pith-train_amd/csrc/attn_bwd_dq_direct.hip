@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_direct_kernel(BwdParams 
   const int kvb0 = HALF ? wave >> 2 : 0;  // the first 32-key block of every tile this wave owns
 
   int m_tile, h, b;
-  decode_block(blockIdx.x, p.Hq, p.B, p.tiles, m_tile, h, b);
+  decode_block(blockIdx.x, p.Hq, p.B, p.tiles, p.group, m_tile, h, b);
   const int hk = h / p.group;
   const int m0 = m_tile * kBM;
   const int q_wave0 = m0 + (HALF ? (wave & 3) : wave) * 32;

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_ds_kernel(BwdParams p) {
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, g = lane >> 5;
   int m_tile, h, b;
-  decode_block(blockIdx.x, p.Hq, p.B, p.tiles, m_tile, h, b);
+  decode_block(blockIdx.x, p.Hq, p.B, p.tiles, p.group, m_tile, h, b);
   const int hk = h / p.group;
   const int m0 = m_tile * kBM;
   const int q_wave0 = m0 + wave * QW;

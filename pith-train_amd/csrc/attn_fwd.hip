@@ -38,7 +38,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_fwd_kernel(FwdParams p) {
   const int c = lane & 31, g = lane >> 5;
 
   int m_tile, h, b;
-  decode_block(blockIdx.x, p.Hq, p.B, p.m_tiles, m_tile, h, b);
+  decode_block(blockIdx.x, p.Hq, p.B, p.m_tiles, p.group, m_tile, h, b);
   const int hk = h / p.group;
   const int m0 = m_tile * BM;
   const int q_wave0 = m0 + wave * ROWS_WAVE;

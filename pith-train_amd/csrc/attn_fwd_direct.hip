@@ -73,7 +73,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
   const int kvb0 = HALF ? (wave >> 2) : 0;  // first 32-key block of a tile this wave owns
 
   int m_tile, h, b;
-  decode_block(blockIdx.x, p.Hq, p.B, p.m_tiles, m_tile, h, b);
+  decode_block(blockIdx.x, p.Hq, p.B, p.m_tiles, p.group, m_tile, h, b);
   const int hk = h / p.group;
   const int m0 = m_tile * kBM;
   const int q_wave0 = m0 + (HALF ? (wave & 3) : wave) * 32;

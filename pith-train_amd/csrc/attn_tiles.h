@@ -85,16 +85,34 @@ __device__ __forceinline__ void wait_all_vector_loads() {
 }
 
 // Maps a linear workgroup id to (tile, head, batch) so that
-//   - tiles are visited from `tiles-1` down to 0 across ALL heads (under a causal mask the late
-//     tiles carry the most work, and the lightest workgroups should be the last ones dispatched);
+//   - tiles are visited from `tiles-1` down to 0 (under a causal mask the late tiles carry the most work, and
+//     the lightest workgroups should be the last ones dispatched);
 //   - workgroups are dealt round-robin to the 8 XCDs of the device, each with its own L2: the
 //     heads of one level are permuted so that an XCD keeps a contiguous range of heads, i.e. the
-//     query heads that share a kv head read their K/V through the same L2.
-__device__ __forceinline__ void decode_block(int linear, int heads, int batch, int tiles, int& tile, int& h, int& b) {
+//     query heads that share a kv head read their K/V through the same L2;
+//   - with more than 8 kv heads per level (`group` = query heads per kv head) and at least kChunkedTiles tiles
+//     the heads are taken in chunks of 8 kv heads, all tiles of a chunk before the next chunk: the workgroups an
+//     XCD holds at one time then belong to ONE kv head and stream the same K/V tiles at about the same time,
+//     instead of one stream per head. Each chunk ends with its light tiles, so the order is no longer
+//     heaviest-first over the whole grid: measured 9-14 % faster at 128 heads x 32768 rows, 2-6 % slower at 4096
+//     rows (16-32 tiles), hence the threshold.
+constexpr int kChunkedTiles = 64;
+__device__ __forceinline__ void decode_block(int linear, int heads, int batch, int tiles, int group, int& tile, int& h, int& b) {
   const int per_level = heads * batch;
-  const int level = linear / per_level;
-  int pos = linear - level * per_level;
-  if ((per_level & 7) == 0) pos = (pos & 7) * (per_level >> 3) + (pos >> 3);
+  const int chunk = 8 * group;
+  int level, pos;
+  if (tiles >= kChunkedTiles && per_level > chunk && per_level % chunk == 0) {
+    const int per_chunk = chunk * tiles;
+    const int c = linear / per_chunk;
+    const int rem = linear - c * per_chunk;
+    level = rem / chunk;
+    const int u = rem - level * chunk;
+    pos = c * chunk + (u & 7) * group + (u >> 3);
+  } else {
+    level = linear / per_level;
+    pos = linear - level * per_level;
+    if ((per_level & 7) == 0) pos = (pos & 7) * (per_level >> 3) + (pos >> 3);
+  }
   tile = tiles - 1 - level;
   b = pos / heads;
   h = pos - b * heads;

@@ -334,7 +334,10 @@ def test_ds_storing_dkdv_kernel_waits_for_its_tile_loads_only(tmp_path_factory):
     text = _kernel_asm("attn_bwd_dkdv_d128.hip", tmp_path_factory.getbasetemp())
     lines = text.splitlines()
     waits = [i for i, l in enumerate(lines) if re.search(r"s_waitcnt vmcnt\(4\)\s*$", l) and "s_barrier" in lines[i + 1]]
-    assert len(waits) == 4, f"expected one steady-state wait per storing kernel variant (2 masks x 2 output types), got {len(waits)}"
+    assert len(waits) == 6, (
+        f"expected one steady-state wait per storing kernel variant (no mask, mask with ascending and with descending "
+        f"query walk; 2 output types each), got {len(waits)}"
+    )
     for w in waits:
         head = max(i for i in range(w) if "Inner Loop Header" in lines[i])
         label = re.match(r"\.(LBB\d+_\d+):", lines[head]).group(1)

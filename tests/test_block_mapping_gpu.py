@@ -96,3 +96,34 @@ def test_descending_query_walk_of_the_causal_dkdv_kernel(gpu):
         H.attn_bwd_dkdv_into(qs, ks, vs, dos, ls, des, dk2, dv2, scale, True)
         _close(dk[:, :, h0 : h0 + 2], dk2, f"dk, kv heads {h0}, {h0 + 1}", tol=1e-2)
         _close(dv[:, :, h0 : h0 + 2], dv2, f"dv, kv heads {h0}, {h0 + 1}", tol=1e-2)
+
+
+def test_chunked_order_with_a_batch_dimension(gpu):
+    """Two batch elements of 8 heads are 16 (batch, head) combinations per tile level: chunked order again, now
+    with a chunk boundary between the batch elements; each element alone (8 combinations) runs in plain order."""
+    Dqk, Dv, B, heads = 128, 128, 2, 8
+    g = torch.Generator().manual_seed(6)
+    scale = Dqk**-0.5
+    q = (torch.randn(B, S, heads, Dqk, generator=g) * scale).to(torch.bfloat16).to(gpu)
+    k = (torch.randn(B, S, heads, Dqk, generator=g) * scale).to(torch.bfloat16).to(gpu)
+    v = (torch.randn(B, S, heads, Dv, generator=g) * scale).to(torch.bfloat16).to(gpu)
+    dout = torch.randn(B, S, heads, Dv, generator=g).to(torch.bfloat16).to(gpu)
+
+    def run(qs, ks, vs, dos):
+        o = torch.full(dos.shape, float("nan"), dtype=torch.bfloat16, device=gpu)
+        lse = torch.full((qs.shape[0], heads, S), float("nan"), device=gpu)
+        H.attn_fwd_into(qs, ks, vs, o, lse, scale, True)
+        delta = torch.empty_like(lse)
+        H.attn_bwd_delta_into(o, dos, delta)
+        dq = torch.full(qs.shape, float("nan"), device=gpu)
+        dk = torch.full(ks.shape, float("nan"), dtype=torch.bfloat16, device=gpu)
+        dv = torch.full(vs.shape, float("nan"), dtype=torch.bfloat16, device=gpu)
+        H.attn_bwd_dkdv_into(qs, ks, vs, dos, lse, delta, dk, dv, scale, True)
+        H.attn_bwd_dq_into(qs, ks, vs, dos, lse, delta, dq, scale, True)
+        return o, dq, dk, dv
+
+    whole = run(q, k, v, dout)
+    for b in range(B):
+        part = run(*(t[b : b + 1] for t in (q, k, v, dout)))
+        for name, w, p in zip(("o", "dq", "dk", "dv"), whole, part):
+            _close(w[b : b + 1], p, f"{name}, batch element {b}")

@@ -1,0 +1,174 @@
+// Probe: would the forward run faster with ONE wavefront per SIMD that owns 64 query rows and all 64 keys of a tile
+// (512 registers per wave; every K / V^T fragment read from LDS feeds two matrix instructions, half the LDS traffic of
+// the shipped kernel), the matrix work of one tile and the softmax of another interleaved inside the single wave?
+// The kernel below runs that loop on tiles that stay in LDS: no global loads, no barriers, no masks, no rescaling,
+// same fragment read patterns (attn_tiles.h), same instruction mix per element as attn_fwd_direct.hip. One workgroup
+// of 4 waves per compute unit. Output: one line per grid size with milliseconds and TFLOP/s (to compare with what the
+// shipped forward reaches inside its loop, global loads and barriers included).
+// Built by tests/probes/build_probes.py, run by tests/test_probes_gpu.py; never part of the library.
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
+#include <cstdint>
+#include <vector>
+#include <cmath>
+#include <cstring>
+#include "attn_tiles.h"
+using namespace pith;
+#define CK(x) do{hipError_t e=(x); if(e!=hipSuccess){printf("HIP error %s at %d\n", hipGetErrorString(e), __LINE__); exit(1);} }while(0)
+
+#ifndef VALU_PER
+#define VALU_PER 3
+#endif
+
+__global__ __launch_bounds__(256) void wide_kernel(const __bf16* __restrict__ src, float* out, int pairs, float kappa) {
+  __shared__ __attribute__((aligned(1024))) char smem[128 * 1024];  // one workgroup per compute unit
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int c = lane & 31, g = lane >> 5;
+  // fill a K tile and a V tile (64 rows x 256 bytes each) with data
+  for (int i = tid; i < 2 * 16384 / 16; i += 256)
+    *reinterpret_cast<u32x4*>(smem + i * 16) = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(src) + i * 16);
+  __syncthreads();
+  const char* kt = smem;
+  const char* vt = smem + 16384;
+  bf16x8 qf[2][8];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+      qf[rb][ks] = *reinterpret_cast<const bf16x8*>(reinterpret_cast<const char*>(src) + 32768 + ((rb * 8 + ks) * 64 + lane) * 16 + (tid >> 6) * 16384);
+  int k_off[8], v_off[4][2];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) k_off[ks] = straight_offset128(c, 2 * ks + g);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) v_off[i][hh] = transposed_offset128(0, hh, 32 * i, lane);
+
+  f32x16 o[2][4];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[rb][i][v] = 0.f;
+  f32x16 sA[2][2], sB[2][2];
+  bf16x8 pA[2][4], pB[2][4];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+    for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) sA[rb][kvb][v] = 0.01f * (v + lane), sB[rb][kvb][v] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pA[rb][j] = qf[rb][j], pB[rb][j] = qf[rb][j + 4];
+  }
+  float l_run[2] = {0.f, 0.f}, mk[2] = {0.5f, 0.25f};
+
+  auto stage = [&](f32x16 (&s_in)[2][2], f32x16 (&s_out)[2][2], bf16x8 (&p_in)[2][4], bf16x8 (&p_out)[2][4]) __attribute__((always_inline)) {
+    bf16x8 av[4][4], ak[8][2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        av[j][i] = lds_read_transposed_at(vt + v_off[i][0] + j * 16 * kRowBytes128, vt + v_off[i][1] + j * 16 * kRowBytes128);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb) ak[ks][kvb] = *reinterpret_cast<const bf16x8*>(kt + k_off[ks] + kvb * 32 * kRowBytes128);
+    // matrix stream: O += V^T P^T of one tile, S^T of another
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) o[rb][i] = mfma32(av[j][i], p_in[rb][j], o[rb][i]);
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s_out[rb][kvb][v] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) s_out[rb][kvb] = mfma32(ak[ks][kvb], qf[rb][ks], s_out[rb][kvb]);
+    // vector stream: softmax of a third tile
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+      float rs = 0.f;
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          s_in[rb][kvb][v] = __builtin_amdgcn_exp2f(s_in[rb][kvb][v] * kappa - mk[rb]);
+          rs += s_in[rb][kvb][v];
+        }
+      l_run[rb] += rs;
+#pragma unroll
+      for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          const f32x16& x = s_in[rb][kvb];
+          p_out[rb][2 * kvb + jj] = to_bf16x8(x[8 * jj], x[8 * jj + 1], x[8 * jj + 2], x[8 * jj + 3], x[8 * jj + 4], x[8 * jj + 5], x[8 * jj + 6], x[8 * jj + 7]);
+        }
+    }
+#ifndef NO_PATTERN
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int m = 0; m < 64; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (m < 40) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER, 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+  };
+  for (int t = 0; t < pairs; ++t) {
+    stage(sA, sB, pA, pB);
+    stage(sB, sA, pB, pA);
+  }
+  float acc = l_run[0] + l_run[1];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc += o[rb][i][v];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc += sA[0][0][v] + sA[1][1][v] + sB[0][1][v] + sB[1][0][v];
+  if (acc == 1.2345f) out[0] = acc;
+}
+
+static uint16_t f2bf(float f) { uint32_t u; memcpy(&u, &f, 4); u += 0x7fff + ((u >> 16) & 1); return u >> 16; }
+
+int main() {
+  const size_t n = (32768 + 4 * 16384) / 2;
+  std::vector<uint16_t> h(n);
+  srand(1);
+  for (size_t i = 0; i < n; ++i) {
+    float u1 = (rand() + 1.0f) / ((float)RAND_MAX + 2.0f), u2 = (rand() + 1.0f) / ((float)RAND_MAX + 2.0f);
+    h[i] = f2bf(0.3f * sqrtf(-2 * logf(u1)) * cosf(6.2831853f * u2));
+  }
+  uint16_t* d; float* out;
+  CK(hipMalloc(&d, n * 2)); CK(hipMalloc(&out, 64));
+  CK(hipMemcpy(d, h.data(), n * 2, hipMemcpyHostToDevice));
+  hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+  const int pairs = 64;  // 128 tiles = 8192 keys
+  for (int grid : {256, 512, 1024}) {
+    for (int rep = 0; rep < 3; ++rep) {
+      hipLaunchKernelGGL(wide_kernel, dim3(grid), dim3(256), 0, 0, (const __bf16*)d, out, pairs, 0.1275f);
+    }
+    CK(hipEventRecord(e0));
+    const int launches = 10;
+    for (int rep = 0; rep < launches; ++rep) hipLaunchKernelGGL(wide_kernel, dim3(grid), dim3(256), 0, 0, (const __bf16*)d, out, pairs, 0.1275f);
+    CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+    float ms; CK(hipEventElapsedTime(&ms, e0, e1)); ms /= launches;
+    const double flop = (double)grid * 4 * (2.0 * pairs) * 64 * 32768.0;
+    printf("wide grid %4d: %.4f ms  %.1f TFLOP/s\n", grid, ms, flop / ms / 1e9);
+  }
+  return 0;
+}

@@ -1,7 +1,8 @@
-"""Runs the two device probes of tests/probes/ (built ahead of time by __graft_entry__.build()) and checks what the
+"""Runs the device probes of tests/probes/ (built ahead of time by __graft_entry__.build()) and checks what the
 design argues from: the full-chip rate of bf16 matrix instructions depends on the operand data and stays below the
 nominal peak with random operands, and fp32 global atomic adds are far too slow to accumulate dQ in a single backward
-kernel. The probes print their tables; profiles/ holds a copy with hardware counters beside it."""
+kernel; and a forward loop with one 64-row wave per SIMD (half the LDS fragment reads) is issue-bound below the
+shipped loop. The probes print their tables; profiles/ holds a copy with hardware counters beside it."""
 
 import os
 import re
@@ -54,3 +55,16 @@ def test_fp32_atomic_rate_is_far_below_what_a_fused_backward_needs(gpu):
     # atomics and the matrix load overlap: together they take about as long as the slower of the two
     alone, both = rows["atomics only, device scope, dkdv mapping"][0], rows["mfma 40 + atomics, device scope"][0]
     assert both < 1.25 * max(alone, rows["mfma only (40 per wave-interval)"][0]), rows
+
+
+def test_one_wide_wave_per_simd_does_not_beat_the_shipped_forward_loop(gpu):
+    rates = []
+    for line in _run("wide_wave_probe"):
+        m = re.match(r"wide grid\s+(\d+):\s+([\d.]+) ms\s+([\d.]+) TFLOP/s", line)
+        if m:
+            rates.append(float(m.group(3)))
+    assert len(rates) == 3, rates
+    # the shipped 128-feature forward sustains about 1400 TFLOP/s inside its loop, with its global tile loads and
+    # barriers; this loop has neither and still stays below that: a single wave cannot issue the softmax of 64 rows
+    # next to 64 matrix instructions per tile fast enough
+    assert all(700 < r < 1400 for r in rates), rates

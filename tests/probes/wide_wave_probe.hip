@@ -17,20 +17,18 @@
 using namespace pith;
 #define CK(x) do{hipError_t e=(x); if(e!=hipSuccess){printf("HIP error %s at %d\n", hipGetErrorString(e), __LINE__); exit(1);} }while(0)
 
-#ifndef VALU_PER
-#define VALU_PER 3
-#endif
-
+// PINNED: the order of the two streams is laid down with scheduling barriers (one matrix instruction, one LDS read, three
+// vector instructions, one exp, repeated); otherwise the compiler's own order.
+template <bool PINNED>
 __global__ __launch_bounds__(256) void wide_kernel(const __bf16* __restrict__ src, float* out, int pairs, float kappa) {
   __shared__ __attribute__((aligned(1024))) char smem[128 * 1024];  // one workgroup per compute unit
   const int tid = threadIdx.x, lane = tid & 63;
   const int c = lane & 31, g = lane >> 5;
-  // fill a K tile and a V tile (64 rows x 256 bytes each) with data
-  for (int i = tid; i < 2 * 16384 / 16; i += 256)
-    *reinterpret_cast<u32x4*>(smem + i * 16) = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(src) + i * 16);
+  // fill four (K tile, V tile) pairs (64 rows x 256 bytes each) with data; the loop walks them like a ring, so
+  // that no fragment read is loop-invariant
+  for (int i = tid; i < 128 * 1024 / 16; i += 256)
+    *reinterpret_cast<u32x4*>(smem + i * 16) = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(src) + (i & 2047) * 16 + (i >> 11) * 64);
   __syncthreads();
-  const char* kt = smem;
-  const char* vt = smem + 16384;
   bf16x8 qf[2][8];
 #pragma unroll
   for (int rb = 0; rb < 2; ++rb)
@@ -65,7 +63,9 @@ __global__ __launch_bounds__(256) void wide_kernel(const __bf16* __restrict__ sr
   }
   float l_run[2] = {0.f, 0.f}, mk[2] = {0.5f, 0.25f};
 
-  auto stage = [&](f32x16 (&s_in)[2][2], f32x16 (&s_out)[2][2], bf16x8 (&p_in)[2][4], bf16x8 (&p_out)[2][4]) __attribute__((always_inline)) {
+  auto stage = [&](int slot, f32x16 (&s_in)[2][2], f32x16 (&s_out)[2][2], bf16x8 (&p_in)[2][4], bf16x8 (&p_out)[2][4]) __attribute__((always_inline)) {
+    const char* kt = smem + (slot & 3) * 32768;
+    const char* vt = kt + 16384;
     bf16x8 av[4][4], ak[8][2];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -115,21 +115,21 @@ __global__ __launch_bounds__(256) void wide_kernel(const __bf16* __restrict__ sr
           p_out[rb][2 * kvb + jj] = to_bf16x8(x[8 * jj], x[8 * jj + 1], x[8 * jj + 2], x[8 * jj + 3], x[8 * jj + 4], x[8 * jj + 5], x[8 * jj + 6], x[8 * jj + 7]);
         }
     }
-#ifndef NO_PATTERN
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+    if constexpr (PINNED) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
-    for (int m = 0; m < 64; ++m) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      if (m < 40) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER, 0);
-      __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+      for (int m = 0; m < 64; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (m < 40) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_barrier(0);
-#endif
   };
   for (int t = 0; t < pairs; ++t) {
-    stage(sA, sB, pA, pB);
-    stage(sB, sA, pB, pA);
+    stage(2 * t, sA, sB, pA, pB);
+    stage(2 * t + 1, sB, sA, pB, pA);
   }
   float acc = l_run[0] + l_run[1];
 #pragma unroll
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void wide_kernel(const __bf16* __restrict__ sr
 static uint16_t f2bf(float f) { uint32_t u; memcpy(&u, &f, 4); u += 0x7fff + ((u >> 16) & 1); return u >> 16; }
 
 int main() {
-  const size_t n = (32768 + 4 * 16384) / 2;
+  const size_t n = (32768 + 4 * 16384 + 4096) / 2;
   std::vector<uint16_t> h(n);
   srand(1);
   for (size_t i = 0; i < n; ++i) {
@@ -158,17 +158,20 @@ int main() {
   CK(hipMemcpy(d, h.data(), n * 2, hipMemcpyHostToDevice));
   hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
   const int pairs = 64;  // 128 tiles = 8192 keys
-  for (int grid : {256, 512, 1024}) {
-    for (int rep = 0; rep < 3; ++rep) {
-      hipLaunchKernelGGL(wide_kernel, dim3(grid), dim3(256), 0, 0, (const __bf16*)d, out, pairs, 0.1275f);
+  for (int pinned = 0; pinned < 2; ++pinned)
+    for (int grid : {256, 512, 1024}) {
+      auto launch = [&]() {
+        if (pinned) hipLaunchKernelGGL(wide_kernel<true>, dim3(grid), dim3(256), 0, 0, (const __bf16*)d, out, pairs, 0.1275f);
+        else hipLaunchKernelGGL(wide_kernel<false>, dim3(grid), dim3(256), 0, 0, (const __bf16*)d, out, pairs, 0.1275f);
+      };
+      for (int rep = 0; rep < 3; ++rep) launch();
+      CK(hipEventRecord(e0));
+      const int launches = 10;
+      for (int rep = 0; rep < launches; ++rep) launch();
+      CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+      float ms; CK(hipEventElapsedTime(&ms, e0, e1)); ms /= launches;
+      const double flop = (double)grid * 4 * (2.0 * pairs) * 64 * 32768.0;
+      printf("wide %s grid %4d: %.4f ms  %.1f TFLOP/s\n", pinned ? "pinned order  " : "compiler order", grid, ms, flop / ms / 1e9);
     }
-    CK(hipEventRecord(e0));
-    const int launches = 10;
-    for (int rep = 0; rep < launches; ++rep) hipLaunchKernelGGL(wide_kernel, dim3(grid), dim3(256), 0, 0, (const __bf16*)d, out, pairs, 0.1275f);
-    CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
-    float ms; CK(hipEventElapsedTime(&ms, e0, e1)); ms /= launches;
-    const double flop = (double)grid * 4 * (2.0 * pairs) * 64 * 32768.0;
-    printf("wide grid %4d: %.4f ms  %.1f TFLOP/s\n", grid, ms, flop / ms / 1e9);
-  }
   return 0;
 }

@@ -414,6 +414,23 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
       __syncthreads();
     }
   };
+  // A merging launch reads 8-16 KB of running output per wave in its epilogue, every compute unit of the device at
+  // the same moment, from memory that nothing has touched since the previous launch. One or two intervals before the
+  // end every lane therefore touches one 128-byte line of its wave's rows (the 4 bytes land in the LDS area behind the
+  // rings, which nobody reads any more), so that the epilogue finds the rows in L2. The loads complete, like the tile
+  // loads, before the wait that ends the next pair of intervals.
+  auto warm_previous_rows = [&]() __attribute__((always_inline)) {
+    if (p.prev_o == nullptr) return;
+    const int row_bytes = p.prev_f32 ? kDv * 4 : kDv * 2;               // 4 or 2 lines per row
+    const int per_row = row_bytes >> 7;
+    const int64_t prev_rs = o_row_stride * (p.prev_f32 ? 4 : 2);
+    const char* base = reinterpret_cast<const char*>(p.prev_o) + (b * p.prev_bs + (int64_t)h * kDv) * (p.prev_f32 ? 4 : 2);
+    char* const dump = smem + kQSpill + wave * 256;
+    for (int idx = lane; idx < 32 * per_row; idx += 64) {  // wave-uniform trip count: 1 or 2
+      const int row = min(q_wave0 + idx / per_row, p.Sq - 1);
+      load_lds4(base + row * prev_rs + (idx % per_row) * 128, dump);
+    }
+  };
   // Every wave passes the same number of barriers; the two roles run separate loops so that
   // each loop body is straight-line code around one accumulator set.
   auto run = [&](auto late_tag) __attribute__((always_inline)) {
@@ -428,6 +445,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_direct_kernel(FwdParams p) 
         interval(i + 1, late_tag, Full{}, std::integral_constant<int, 2>{});
       }
     }
+    if constexpr (kQViaLds && !CAUSAL) warm_previous_rows();
     for (; i + 1 < n_tiles_wave; ++i) interval(i, late_tag, Full{}, std::integral_constant<int, 0>{});
     for (; i < n_tiles_wg; ++i) interval(i, late_tag, Part{}, std::integral_constant<int, 0>{});
   };
